@@ -1,0 +1,166 @@
+/*
+ * ltr_attn.h - C ABI of the MI355X (gfx950) ring / block attention library.
+ *
+ * The reference (lwj2015/lightron) is pure Python and has no FFI; each entry point
+ * below names the reference code whose arithmetic it replaces.  A binder needs only
+ * this header: plain pointers, sizes, no C++ or torch types.  All pointers are DEVICE
+ * pointers unless noted.  Every call enqueues work on `stream` (a hipStream_t passed
+ * as void*; NULL = the default stream) of the CURRENT device and returns without
+ * synchronising.  The library never allocates, frees or keeps a pointer after the
+ * call returns; all buffers, including fp32 gradient accumulators, belong to the
+ * caller.  Return value: 0 on success, a negative LTR_E* code otherwise (nothing is
+ * enqueued on error).  Re-entrant; no mutable global state.
+ *
+ * Tensor layout: element strides (in elements, not bytes) are given for the batch,
+ * sequence and head dimensions; the head dimension D is contiguous.  This serves
+ * [B,S,H,D] (the layout at every reference boundary, ring_attention.py:13),
+ * [B,H,S,D] (the layout at the SDPA call sites) and the Ulysses head-slice view
+ * (parallel_cp.py:206-208) without copies.  LSE and DELTA are fp32 [B, Hq, Sq]
+ * contiguous.
+ *
+ * Positions: query row i of the local chunk has global position
+ *     i <  q_split : q_pos0[0] + i
+ *     i >= q_split : q_pos0[1] + (i - q_split)
+ * (q_split = Sq for one contiguous chunk; the two-segment form is the zig-zag
+ * assignment).  Key row j of KV chunk c has global position chunk[c].pos0 + j.
+ * With LTR_CAUSAL a key is visible iff key_pos <= query_pos.  Rows with no visible
+ * key get O = 0 and LSE = -inf.
+ */
+#ifndef LTR_ATTN_H
+#define LTR_ATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LTR_ABI_VERSION 1
+#define LTR_MAX_CHUNKS 32
+
+/* element types */
+#define LTR_BF16 0
+#define LTR_F32 1
+
+/* flags */
+#define LTR_CAUSAL 1u /* mask by global position */
+#define LTR_MERGE 2u  /* forward: o/lse hold an earlier partial result; merge into it */
+
+/* error codes */
+#define LTR_OK 0
+#define LTR_EINVAL (-1)   /* null pointer, bad size, bad flag */
+#define LTR_EUNSUP (-2)   /* unsupported head dim / dtype combination */
+#define LTR_EALIGN (-3)   /* pointer or stride not 16-byte aligned */
+#define LTR_ELAUNCH (-4)  /* HIP reported a launch error */
+#define LTR_EDEVICE (-5)  /* current device is not gfx950 */
+
+typedef struct ltr_kv_chunk {
+    const void *k; /* [B, sk, Hkv, D] by kv strides */
+    const void *v;
+    void *dk;      /* fp32 accumulators, same logical shape, by dkv strides (backward only) */
+    void *dv;
+    int64_t sk;    /* keys in this chunk */
+    int64_t pos0;  /* global position of its first key */
+} ltr_kv_chunk;
+
+/*
+ * ltr_attn_fwd - one rank's local Q chunk attended against n_chunks KV chunks resident
+ * in HBM, online softmax across chunks kept in registers, O normalised and LSE written
+ * once.  Replaces the whole `for step in range(world_size)` body of
+ * ring_attention_kernel (parallel/communication/ring_attention.py:46-118: score GEMM
+ * :71, online-softmax update :79-95/:107, PV GEMM and rescale :101-104, normalise :118)
+ * and the SDPA calls at parallel/parallel_cp.py:224-229 and model/model.py:193-198.
+ * GQA: q head h reads kv head h / (Hq/Hkv)  (model/model.py:11-34, repeat_kv).
+ * With LTR_MERGE the epilogue combines the new partial (O', LSE') with the (O, LSE)
+ * already in the output buffers by the same rule
+ *     LSE = logaddexp(LSE, LSE'),  O = O*exp(LSE_old-LSE) + O'*exp(LSE'-LSE)
+ * so a caller that receives KV chunks one at a time (one launch per ring step, as at
+ * ring_attention.py:46) needs no separate merge pass.
+ */
+typedef struct ltr_attn_fwd_args {
+    const void *q;      /* [B, Sq, Hq, D] by q strides; dtype io_dtype */
+    void *o;            /* same logical shape by o strides; dtype o_dtype */
+    float *lse;         /* [B, Hq, Sq] */
+    int32_t B, Hq, Hkv, D; /* D in {64, 128} */
+    int64_t Sq;
+    int64_t q_stride[3];  /* batch, seq, head */
+    int64_t o_stride[3];
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t q_pos0[2];
+    int64_t q_split;
+    float scale;          /* 1/sqrt(D) at every reference call site (ring_attention.py:20) */
+    uint32_t flags;
+    int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v */
+    int32_t o_dtype;      /* LTR_BF16 or LTR_F32 */
+    int32_t n_chunks;     /* 1..LTR_MAX_CHUNKS */
+    ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
+} ltr_attn_fwd_args;
+
+int ltr_attn_fwd(const ltr_attn_fwd_args *args, void *stream);
+
+/*
+ * ltr_attn_bwd_delta - DELTA[b,h,i] = sum_d dO[b,i,h,d] * O[b,i,h,d], the row term of
+ * the softmax Jacobian.  The reference has no hand-written backward (autograd through
+ * ring_attention.py:66-118 / SDPA); this is the first stage of the recompute backward.
+ */
+typedef struct ltr_attn_delta_args {
+    const void *o;
+    const void *d_o;
+    float *delta;       /* [B, Hq, Sq] */
+    int32_t B, Hq, D;
+    int64_t Sq;
+    int64_t o_stride[3];
+    int64_t do_stride[3];
+    int32_t o_dtype;    /* dtype of o */
+    int32_t do_dtype;   /* dtype of dO */
+} ltr_attn_delta_args;
+
+int ltr_attn_bwd_delta(const ltr_attn_delta_args *args, void *stream);
+
+/*
+ * ltr_attn_bwd - recompute backward of ltr_attn_fwd for the same Q chunk / KV chunk
+ * table: P = exp(S*scale - LSE), dV += P^T dO, dP = dO V^T, dS = P*(dP - DELTA),
+ * dQ += dS K * scale, dK += dS^T Q * scale.  Replaces torch autograd through the ring
+ * body / SDPA (trainer.py:54 -> parallel_cp.py:224-229).  dq, chunk[c].dk and
+ * chunk[c].dv are fp32 ACCUMULATORS: the caller zero-fills them before the first
+ * launch that contributes, launches on one stream accumulate (that is how dK/dV sum
+ * over the Q chunks of several ranks), and ltr_cast_f32_to_bf16 makes the final cast.
+ * dK/dV of a GQA group sum over its Hq/Hkv query heads.
+ */
+typedef struct ltr_attn_bwd_args {
+    const void *q;
+    const void *d_o;      /* same dtype as q */
+    const float *lse;     /* [B, Hq, Sq], of the COMPLETE softmax (all chunks) */
+    const float *delta;   /* [B, Hq, Sq] */
+    float *dq;            /* fp32 accumulator, by dq strides */
+    int32_t B, Hq, Hkv, D;
+    int64_t Sq;
+    int64_t q_stride[3];
+    int64_t do_stride[3];
+    int64_t dq_stride[3];
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t dk_stride[3];
+    int64_t dv_stride[3];
+    int64_t q_pos0[2];
+    int64_t q_split;
+    float scale;
+    uint32_t flags;       /* LTR_CAUSAL */
+    int32_t io_dtype;     /* LTR_BF16 or LTR_F32 */
+    int32_t n_chunks;
+    ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
+} ltr_attn_bwd_args;
+
+int ltr_attn_bwd(const ltr_attn_bwd_args *args, void *stream);
+
+/* dst[i] = bf16(src[i]) (round to nearest even), i < n; both contiguous. */
+int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream);
+
+int ltr_abi_version(void);
+const char *ltr_strerror(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LTR_ATTN_H */

@@ -1,0 +1,93 @@
+"""ctypes binding of include/ltr_attn.h.  No fallback: if the shared library is missing the
+import of any compute entry point raises, and a GPU call on a non-gfx950 device returns
+LTR_EDEVICE from the library."""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
+
+LTR_ABI_VERSION = 1
+LTR_MAX_CHUNKS = 32
+LTR_BF16, LTR_F32 = 0, 1
+LTR_CAUSAL, LTR_MERGE = 1, 2
+
+EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16",
+           "ltr_abi_version", "ltr_strerror")
+
+_i64x3 = ctypes.c_int64 * 3
+_i64x2 = ctypes.c_int64 * 2
+
+
+class KvChunk(ctypes.Structure):
+    _fields_ = [("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("dk", ctypes.c_void_p), ("dv", ctypes.c_void_p),
+                ("sk", ctypes.c_int64), ("pos0", ctypes.c_int64)]
+
+
+class FwdArgs(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("o", ctypes.c_void_p), ("lse", ctypes.c_void_p),
+                ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("D", ctypes.c_int32),
+                ("Sq", ctypes.c_int64),
+                ("q_stride", _i64x3), ("o_stride", _i64x3), ("k_stride", _i64x3), ("v_stride", _i64x3),
+                ("q_pos0", _i64x2), ("q_split", ctypes.c_int64),
+                ("scale", ctypes.c_float), ("flags", ctypes.c_uint32),
+                ("io_dtype", ctypes.c_int32), ("o_dtype", ctypes.c_int32), ("n_chunks", ctypes.c_int32),
+                ("chunk", KvChunk * LTR_MAX_CHUNKS)]
+
+
+class DeltaArgs(ctypes.Structure):
+    _fields_ = [("o", ctypes.c_void_p), ("d_o", ctypes.c_void_p), ("delta", ctypes.c_void_p),
+                ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("D", ctypes.c_int32),
+                ("Sq", ctypes.c_int64),
+                ("o_stride", _i64x3), ("do_stride", _i64x3),
+                ("o_dtype", ctypes.c_int32), ("do_dtype", ctypes.c_int32)]
+
+
+class BwdArgs(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("d_o", ctypes.c_void_p), ("lse", ctypes.c_void_p),
+                ("delta", ctypes.c_void_p), ("dq", ctypes.c_void_p),
+                ("B", ctypes.c_int32), ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("D", ctypes.c_int32),
+                ("Sq", ctypes.c_int64),
+                ("q_stride", _i64x3), ("do_stride", _i64x3), ("dq_stride", _i64x3),
+                ("k_stride", _i64x3), ("v_stride", _i64x3), ("dk_stride", _i64x3), ("dv_stride", _i64x3),
+                ("q_pos0", _i64x2), ("q_split", ctypes.c_int64),
+                ("scale", ctypes.c_float), ("flags", ctypes.c_uint32),
+                ("io_dtype", ctypes.c_int32), ("n_chunks", ctypes.c_int32),
+                ("chunk", KvChunk * LTR_MAX_CHUNKS)]
+
+
+_lib = None
+
+
+def load():
+    """Load (once) and return the ctypes handle; raises if the extension has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "lightron_amd: %s is missing - build it with `python -m lightron_amd.build` "
+            "(there is no CPU or PyTorch fallback)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.ltr_attn_fwd.argtypes = [ctypes.POINTER(FwdArgs), ctypes.c_void_p]
+    lib.ltr_attn_fwd.restype = ctypes.c_int
+    lib.ltr_attn_bwd_delta.argtypes = [ctypes.POINTER(DeltaArgs), ctypes.c_void_p]
+    lib.ltr_attn_bwd_delta.restype = ctypes.c_int
+    lib.ltr_attn_bwd.argtypes = [ctypes.POINTER(BwdArgs), ctypes.c_void_p]
+    lib.ltr_attn_bwd.restype = ctypes.c_int
+    lib.ltr_cast_f32_to_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    lib.ltr_cast_f32_to_bf16.restype = ctypes.c_int
+    lib.ltr_abi_version.argtypes = []
+    lib.ltr_abi_version.restype = ctypes.c_int
+    lib.ltr_strerror.argtypes = [ctypes.c_int]
+    lib.ltr_strerror.restype = ctypes.c_char_p
+    if lib.ltr_abi_version() != LTR_ABI_VERSION:
+        raise RuntimeError("lightron_amd: ABI version mismatch (library %d, binding %d)"
+                           % (lib.ltr_abi_version(), LTR_ABI_VERSION))
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        raise RuntimeError("%s failed: %s (%d)" % (what, load().ltr_strerror(rc).decode(), rc))

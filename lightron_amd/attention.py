@@ -1,0 +1,220 @@
+"""Host side of the block-attention C ABI: argument marshalling and the autograd Function.
+
+Tensors are logical [B, S, H, D] with arbitrary batch/seq/head strides and a contiguous
+last dim, so [B,H,S,D] storage (pass ``x.transpose(1, 2)``) and head-slice views work
+without copies.  All compute happens in the HIP library; there is no PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+
+_DT = {torch.bfloat16: _lib.LTR_BF16, torch.float32: _lib.LTR_F32}
+
+
+def _stream_ptr(dev) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _s3(t: torch.Tensor):
+    return (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _req(t: torch.Tensor, name: str):
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a GPU tensor (the HIP library has no CPU path)" % name)
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise RuntimeError("%s must be [B,S,H,D] with a contiguous last dim, got shape %s strides %s"
+                           % (name, tuple(t.shape), t.stride()))
+
+
+def _same_strides(ts: Sequence[torch.Tensor]) -> bool:
+    s0 = ts[0].stride()
+    return all(t.stride() == s0 for t in ts)
+
+
+def _norm_chunks(ks, vs):
+    """The ABI carries one stride triple for all K chunks and one for all V chunks."""
+    if not _same_strides(ks):
+        ks = [k.contiguous() for k in ks]
+    if not _same_strides(vs):
+        vs = [v.contiguous() for v in vs]
+    return list(ks), list(vs)
+
+
+def _qpos(q_pos0, Sq, q_split):
+    if isinstance(q_pos0, int):
+        q_pos0 = (q_pos0, q_pos0)
+    if q_split is None:
+        q_split = Sq
+    return (ctypes.c_int64 * 2)(int(q_pos0[0]), int(q_pos0[1])), int(q_split)
+
+
+def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Tensor], k_pos0: Sequence[int],
+             q_pos0=0, q_split: Optional[int] = None, causal: bool = False, scale: Optional[float] = None,
+             out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None, merge: bool = False,
+             out_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One Q chunk against a table of KV chunks -> (O [B,Sq,Hq,D], LSE [B,Hq,Sq] fp32).
+    With merge=True, `out`/`lse` hold an earlier partial result which is merged in place."""
+    lib = _lib.load()
+    _req(q, "q")
+    B, Sq, Hq, D = q.shape
+    ks, vs = _norm_chunks(ks, vs)
+    for k, v in zip(ks, vs):
+        _req(k, "k")
+        _req(v, "v")
+        if k.dtype != q.dtype or v.dtype != q.dtype or k.shape != v.shape or k.shape[0] != B or k.shape[3] != D:
+            raise RuntimeError("k/v chunk shape or dtype mismatch")
+    Hkv = ks[0].shape[2]
+    if q.dtype not in _DT:
+        raise RuntimeError("unsupported dtype %s" % q.dtype)
+    if out is None:
+        if merge:
+            raise RuntimeError("merge=True needs the earlier partial result in out/lse")
+        out = torch.empty((B, Sq, Hq, D), dtype=out_dtype or q.dtype, device=q.device)
+        lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    _req(out, "out")
+    if lse is None or lse.dtype != torch.float32 or not lse.is_contiguous() or tuple(lse.shape) != (B, Hq, Sq):
+        raise RuntimeError("lse must be a contiguous fp32 [B,Hq,Sq] tensor")
+    a = _lib.FwdArgs()
+    a.q, a.o, a.lse = q.data_ptr(), out.data_ptr(), lse.data_ptr()
+    a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, Hkv, D, Sq
+    a.q_stride, a.o_stride = _s3(q), _s3(out)
+    a.k_stride, a.v_stride = _s3(ks[0]), _s3(vs[0])
+    a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
+    a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
+    a.io_dtype, a.o_dtype = _DT[q.dtype], _DT[out.dtype]
+    stream = _stream_ptr(q.device)
+    n = len(ks)
+    with torch.cuda.device(q.device):
+        for start in range(0, n, _lib.LTR_MAX_CHUNKS):
+            stop = min(n, start + _lib.LTR_MAX_CHUNKS)
+            a.n_chunks = stop - start
+            for i in range(start, stop):
+                ch = a.chunk[i - start]
+                ch.k, ch.v, ch.dk, ch.dv = ks[i].data_ptr(), vs[i].data_ptr(), None, None
+                ch.sk, ch.pos0 = ks[i].shape[1], int(k_pos0[i])
+            a.flags = (_lib.LTR_CAUSAL if causal else 0) | (_lib.LTR_MERGE if (merge or start > 0) else 0)
+            _lib.check(lib.ltr_attn_fwd(ctypes.byref(a), stream), "ltr_attn_fwd")
+    return out, lse
+
+
+def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
+    lib = _lib.load()
+    _req(o, "o")
+    _req(do, "dO")
+    B, Sq, Hq, D = o.shape
+    delta = torch.empty((B, Hq, Sq), dtype=torch.float32, device=o.device)
+    a = _lib.DeltaArgs()
+    a.o, a.d_o, a.delta = o.data_ptr(), do.data_ptr(), delta.data_ptr()
+    a.B, a.Hq, a.D, a.Sq = B, Hq, D, Sq
+    a.o_stride, a.do_stride = _s3(o), _s3(do)
+    a.o_dtype, a.do_dtype = _DT[o.dtype], _DT[do.dtype]
+    with torch.cuda.device(o.device):
+        _lib.check(lib.ltr_attn_bwd_delta(ctypes.byref(a), _stream_ptr(o.device)), "ltr_attn_bwd_delta")
+    return delta
+
+
+def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
+                        causal=False, scale=None):
+    """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs."""
+    lib = _lib.load()
+    _req(q, "q")
+    _req(do, "dO")
+    B, Sq, Hq, D = q.shape
+    ks, vs = _norm_chunks(ks, vs)
+    if not (_same_strides(dk_accs) and _same_strides(dv_accs)):
+        raise RuntimeError("dk/dv accumulators must share one stride triple each")
+    for t in [dq_acc] + list(dk_accs) + list(dv_accs):
+        _req(t, "accumulator")
+        if t.dtype != torch.float32:
+            raise RuntimeError("gradient accumulators must be fp32")
+    a = _lib.BwdArgs()
+    a.q, a.d_o, a.lse, a.delta, a.dq = q.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(), dq_acc.data_ptr()
+    a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, ks[0].shape[2], D, Sq
+    a.q_stride, a.do_stride, a.dq_stride = _s3(q), _s3(do), _s3(dq_acc)
+    a.k_stride, a.v_stride = _s3(ks[0]), _s3(vs[0])
+    a.dk_stride, a.dv_stride = _s3(dk_accs[0]), _s3(dv_accs[0])
+    a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
+    a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
+    a.flags = _lib.LTR_CAUSAL if causal else 0
+    a.io_dtype = _DT[q.dtype]
+    stream = _stream_ptr(q.device)
+    n = len(ks)
+    with torch.cuda.device(q.device):
+        for start in range(0, n, _lib.LTR_MAX_CHUNKS):
+            stop = min(n, start + _lib.LTR_MAX_CHUNKS)
+            a.n_chunks = stop - start
+            for i in range(start, stop):
+                ch = a.chunk[i - start]
+                ch.k, ch.v = ks[i].data_ptr(), vs[i].data_ptr()
+                ch.dk, ch.dv = dk_accs[i].data_ptr(), dv_accs[i].data_ptr()
+                ch.sk, ch.pos0 = ks[i].shape[1], int(k_pos0[i])
+            _lib.check(lib.ltr_attn_bwd(ctypes.byref(a), stream), "ltr_attn_bwd")
+
+
+def cast_to_bf16(src: torch.Tensor) -> torch.Tensor:
+    lib = _lib.load()
+    if src.dtype != torch.float32 or not src.is_contiguous():
+        raise RuntimeError("cast_to_bf16 needs a contiguous fp32 tensor")
+    dst = torch.empty(src.shape, dtype=torch.bfloat16, device=src.device)
+    with torch.cuda.device(src.device):
+        _lib.check(lib.ltr_cast_f32_to_bf16(src.data_ptr(), dst.data_ptr(), src.numel(), _stream_ptr(src.device)),
+                   "ltr_cast_f32_to_bf16")
+    return dst
+
+
+class BlockAttentionFunction(torch.autograd.Function):
+    """O = attention(q ; KV chunk table) with the recompute backward.  Inputs after the
+    fixed arguments are k_0..k_{n-1}, v_0..v_{n-1}."""
+
+    @staticmethod
+    def forward(ctx, q, n_chunks, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, *kv):
+        ks, vs = list(kv[:n_chunks]), list(kv[n_chunks:])
+        if stepwise:
+            # one launch per KV chunk, merged in the epilogue into an fp32 running (O, LSE)
+            o, lse = attn_fwd(q, ks[:1], vs[:1], k_pos0[:1], q_pos0, q_split, causal, scale, out_dtype=torch.float32)
+            for i in range(1, n_chunks):
+                attn_fwd(q, ks[i:i + 1], vs[i:i + 1], k_pos0[i:i + 1], q_pos0, q_split, causal, scale,
+                         out=o, lse=lse, merge=True)
+            if (out_dtype or q.dtype) != torch.float32:
+                o = o.to(out_dtype or q.dtype)
+        else:
+            o, lse = attn_fwd(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, out_dtype=out_dtype)
+        ctx.save_for_backward(q, o, lse, *kv)
+        ctx.meta = (n_chunks, list(k_pos0), q_pos0, q_split, causal, scale)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, _dlse):
+        q, o, lse, *kv = ctx.saved_tensors
+        n_chunks, k_pos0, q_pos0, q_split, causal, scale = ctx.meta
+        ks, vs = kv[:n_chunks], kv[n_chunks:]
+        if q.dtype != torch.bfloat16:
+            raise RuntimeError("the HIP backward is implemented for bf16 inputs")
+        if do.stride(3) != 1:
+            do = do.contiguous()
+        do = do.to(q.dtype)
+        delta = attn_delta(o, do)
+        dq_acc = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        dk_accs = [torch.zeros(k.shape, dtype=torch.float32, device=q.device) for k in ks]
+        dv_accs = [torch.zeros(v.shape, dtype=torch.float32, device=q.device) for v in vs]
+        attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale)
+        dq = cast_to_bf16(dq_acc)
+        dks = [cast_to_bf16(x) for x in dk_accs]
+        dvs = [cast_to_bf16(x) for x in dv_accs]
+        return (dq, None, None, None, None, None, None, None, None, *dks, *dvs)
+
+
+def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, scale=None, stepwise=False,
+                    out_dtype=None):
+    """Differentiable entry: returns (O, LSE)."""
+    n = len(ks)
+    return BlockAttentionFunction.apply(q, n, list(k_pos0), q_pos0, q_split, causal, scale, stepwise, out_dtype,
+                                        *ks, *vs)

@@ -1,0 +1,34 @@
+"""Build recipe for the HIP extension: one hipcc call, gfx950 only, output in-tree."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SRC = os.path.join(HERE, "csrc", "ltr_attn.hip")
+LIB = os.path.join(HERE, "csrc", "libltr_attn.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-shared", "-fPIC", "-std=c++17",
+    "-munsafe-fp-atomics",                      # hardware global_atomic_add_f32 for the dQ accumulator
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I", os.path.join(ROOT, "include"),
+]
+
+
+def build(verbose: bool = False) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    if not os.path.exists(hipcc):
+        hipcc = "hipcc"
+    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB, SRC]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed building %s" % SRC)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,975 @@
+// Ring / block attention for MI355X (gfx950, CDNA4): forward with online softmax across
+// KV chunks resident in HBM, recompute backward, behind the C ABI of include/ltr_attn.h.
+//
+// Kernel map
+//   fwd_bf16_kernel<D>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a wave
+//                        owns 32 query rows, so a lane owns ONE query: the row max / sum are
+//                        in-lane reductions plus one v_permlane32_swap, and P^T leaves the
+//                        first GEMM already in the B-operand layout of the second.  K and V
+//                        tiles are staged in LDS by 128-bit loads; the V^T operand is read
+//                        with ds_read_b64_tr_b16.  The (O, LSE) merge with an earlier partial
+//                        result is part of the epilogue.
+//   fwd_f32_kernel<D>    fp32 I/O and arithmetic (no MFMA), for the 1e-4 parity case.
+//   delta_kernel         DELTA = rowsum(dO * O).
+//   bwd_bf16_kernel<D>   a block owns 128 keys of one kv head (32 per wave, K and V operands
+//                        resident in registers), loops over the query heads of the GQA group
+//                        and over query tiles; dK^T/dV^T accumulate in registers, dS goes
+//                        through LDS so each wave forms a complete 32x32 slice of dQ, which is
+//                        added to the fp32 accumulator in HBM with hardware float atomics.
+//
+// MFMA 32x32x16 operand layout used throughout (lane l, i = l % 32, h = l / 32):
+//   A[i][8h .. 8h+7], B[8h .. 8h+7][i], C[8*(r/4) + 4h + r%4][i] for accumulator register r.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+#include "ltr_attn.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+
+#define LTR_LOG2E 1.4426950408889634f
+#define LTR_LN2 0.6931471805599453f
+
+struct ChunkDev {
+    const void *k;
+    const void *v;
+    float *dk;
+    float *dv;
+    int sk;
+    int pos0;
+};
+
+struct FwdParams {
+    const void *q;
+    void *o;
+    float *lse;
+    int B, Hq, Hkv, n_rep;
+    int Sq, n_qtiles;
+    long long qs[3], os[3], ks[3], vs[3];
+    int q_pos0[2];
+    int q_split;
+    float scale;
+    unsigned flags;
+    int o_f32;
+    int n_chunks;
+    ChunkDev chunk[LTR_MAX_CHUNKS];
+};
+
+struct BwdParams {
+    const void *q;
+    const void *d_o;
+    const float *lse;
+    const float *delta;
+    float *dq;
+    int B, Hq, Hkv, n_rep;
+    int Sq, n_qtiles;
+    long long qs[3], dos[3], dqs[3], ks[3], vs[3], dks[3], dvs[3];
+    int q_pos0[2];
+    int q_split;
+    float scale;
+    unsigned flags;
+    int n_chunks;
+    int tiles_total;  // key tiles over all chunks
+    ChunkDev chunk[LTR_MAX_CHUNKS];
+};
+
+struct DeltaParams {
+    const void *o;
+    const void *d_o;
+    float *delta;
+    int B, Hq, D, Sq;
+    long long os[3], dos[3];
+    int o_f32, do_f32;
+};
+
+__device__ __forceinline__ int q_position(int row, int split, int p0, int p1) {
+    return row < split ? p0 + row : p1 + (row - split);
+}
+
+// min and max global position over local rows [r0, r1] (inclusive, r0 <= r1)
+__device__ __forceinline__ void q_pos_range(int r0, int r1, int split, int p0, int p1, int &lo, int &hi) {
+    int a = q_position(r0, split, p0, p1), b = q_position(r1, split, p0, p1);
+    lo = min(a, b);
+    hi = max(a, b);
+    if (r0 < split && r1 >= split) {  // tile straddles the two segments
+        int c = q_position(split - 1, split, p0, p1), d = q_position(split, split, p0, p1);
+        lo = min(lo, min(c, d));
+        hi = max(hi, max(c, d));
+    }
+}
+
+// both halves of the wave end up with combine(x[l], x[l ^ 32])
+__device__ __forceinline__ float xhalf_max(float x) {
+    unsigned u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xhalf_sum(float x) {
+    unsigned u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives as element e the
+// 16-bit value that lane (4e + i/4) of the group addressed at position i % 4.  With lane s
+// of a group pointing at M[k0 + s/4][n0 + 4*(s%4)] of a row-major tile, lane i receives
+// M[k0 + 0..3][n0 + i]: four consecutive rows of one column, i.e. the MFMA K-dim packing.
+__device__ __forceinline__ i16x4 lds_read_tr16(const __bf16 *p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)(p));
+}
+
+// 8 K-dim values for an MFMA operand whose K index runs over the ROWS of a row-major LDS
+// tile: rows {k0 + 4h + 0..3} and {k0 + 8 + 4h + 0..3} at column n_base + (l % 32).
+// This row set is the one the accumulator registers 8b..8b+7 of a 32x32 MFMA result
+// hold (rows 16b + 4h + 0..3 and 16b + 8 + 4h + 0..3), so a result tile can feed the
+// next GEMM as an operand without leaving registers.
+__device__ __forceinline__ bf16x8 lds_operand_tr(const __bf16 *tile, int stride, int k0, int n_base, int lane) {
+    const int li = lane & 15, g = lane >> 4;
+    const int hh = g >> 1;
+    const int col = n_base + ((g & 1) << 4) + ((li & 3) << 2);
+    const int row = k0 + 4 * hh + (li >> 2);
+    i16x4 lo = lds_read_tr16(tile + row * stride + col);
+    i16x4 hi = lds_read_tr16(tile + (row + 8) * stride + col);
+    union {
+        struct { i16x4 a, b; } s;
+        bf16x8 v;
+    } u;
+    u.s.a = lo;
+    u.s.b = hi;
+    return u.v;
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) {
+    union { uint4 u; bf16x8 v; } c;
+    c.u = x;
+    return c.v;
+}
+
+__device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16 &s, int base) {
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; e++) r[e] = (__bf16)s[base + e];
+    return r;
+}
+
+// ------------------------------------------------------------------------------ forward, bf16
+template <int D>
+__global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdParams p) {
+    constexpr int BM = 128, BN = 64;
+    constexpr int KS = D + 8;    // K tile row stride (elements): natural 128-bit operand reads
+    constexpr int VS = D + 16;   // V tile row stride: transpose reads
+    constexpr int CPR = D / 8;   // 16-byte chunks per row
+    constexpr int NLD = BN * CPR / 256;
+    __shared__ __attribute__((aligned(16))) __bf16 Ks[BN * KS];
+    __shared__ __attribute__((aligned(16))) __bf16 Vs[BN * VS];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const bool causal = p.flags & LTR_CAUSAL;
+
+    // block -> (batch, kv head, q head of the group, q tile).  Consecutive block ids go to
+    // the 8 XCDs round-robin; keep all q tiles / q heads of one (batch, kv head) on one XCD
+    // so its K/V stay in that XCD's L2.  Late (heavier under a causal mask) q tiles first.
+    int idx = blockIdx.x, pair, rest;
+    const int P = p.B * p.Hkv;
+    if ((P & 7) == 0) {
+        int xcd = idx & 7, j = idx >> 3, pp = P >> 3;
+        pair = (j % pp) * 8 + xcd;
+        rest = j / pp;
+    } else {
+        pair = idx % P;
+        rest = idx / P;
+    }
+    const int rep = rest % p.n_rep;
+    const int qt = p.n_qtiles - 1 - rest / p.n_rep;
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
+
+    const int row0 = qt * BM;
+    const int my_row = row0 + w * 32 + l32;
+    const bool row_ok = my_row < p.Sq;
+    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int blk_lo, blk_hi, w_lo, w_hi;
+    q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+    {
+        int wr0 = row0 + w * 32, wr1 = min(wr0 + 32, p.Sq) - 1;
+        if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
+        else { w_lo = 0x7fffffff; w_hi = -0x7fffffff; }  // wave has no valid row
+    }
+
+    // Q operand (B of S^T = K Q^T): lane (query l32, half hh) holds d = 16*kb + 8*hh .. +7
+    bf16x8 qreg[D / 16];
+    {
+        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + (long long)my_row * p.qs[1] + h * p.qs[2];
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) {
+            uint4 x = make_uint4(0, 0, 0, 0);
+            if (row_ok) x = *(const uint4 *)(qp + kb * 16 + 8 * hh);
+            qreg[kb] = as_bf16x8(x);
+        }
+    }
+
+    f32x16 oacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
+    float m_run = -INFINITY;  // running max of raw scores (before scale)
+    float l_run = 0.f;        // this lane's partial row sum (its 32 of the 64 keys per tile)
+    const float c2 = p.scale * LTR_LOG2E;
+
+    // tile iterator over (chunk, key tile)
+    int c = 0, t = 0, nt = 0;
+    auto ntiles_of = [&](int ci) {
+        int sk = p.chunk[ci].sk;
+        int nvis = causal ? max(0, min(sk, blk_hi - p.chunk[ci].pos0 + 1)) : sk;
+        return (nvis + BN - 1) / BN;
+    };
+    auto settle = [&]() {
+        while (c < p.n_chunks && t >= nt) {
+            c++;
+            t = 0;
+            if (c < p.n_chunks) nt = ntiles_of(c);
+        }
+    };
+    nt = ntiles_of(0);
+    settle();
+
+    uint4 kld[NLD], vld[NLD];
+    auto gload = [&](int ci, int ti) {
+        const __bf16 *kp = (const __bf16 *)p.chunk[ci].k + b * p.ks[0] + hkv * p.ks[2];
+        const __bf16 *vp = (const __bf16 *)p.chunk[ci].v + b * p.vs[0] + hkv * p.vs[2];
+        const int sk = p.chunk[ci].sk;
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            int id = tid + 256 * i;
+            int key = ti * BN + id / CPR, dc = id % CPR;
+            kld[i] = make_uint4(0, 0, 0, 0);
+            vld[i] = make_uint4(0, 0, 0, 0);
+            if (key < sk) {
+                kld[i] = *(const uint4 *)(kp + (long long)key * p.ks[1] + dc * 8);
+                vld[i] = *(const uint4 *)(vp + (long long)key * p.vs[1] + dc * 8);
+            }
+        }
+    };
+
+    bool have = c < p.n_chunks;
+    if (have) gload(c, t);
+    while (have) {
+        const int cc = c, ct = t;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            int id = tid + 256 * i;
+            int key = id / CPR, dc = id % CPR;
+            *(uint4 *)(Ks + key * KS + dc * 8) = kld[i];
+            *(uint4 *)(Vs + key * VS + dc * 8) = vld[i];
+        }
+        __syncthreads();
+        t++;
+        settle();
+        const bool have_next = c < p.n_chunks;
+        if (have_next) gload(c, t);
+
+        const int sk = p.chunk[cc].sk, pos0 = p.chunk[cc].pos0;
+        const int key0 = ct * BN;
+        // wave-uniform: does this wave see any key of the tile at all?
+        const bool wave_active = !causal || (pos0 + key0 <= w_hi);
+        if (wave_active) {
+            f32x16 s[2];
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[nb][r] = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < D / 16; kb++) {
+                    bf16x8 a = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
+                    s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
+                }
+            }
+            const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
+            if (need_mask) {
+#pragma unroll
+                for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                        bool vis = key < sk && (!causal || pos0 + key <= my_pos);
+                        if (!vis) s[nb][r] = -INFINITY;
+                    }
+            }
+            float mx = s[0][0];
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[nb][r]);
+            mx = xhalf_max(mx);
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = exp2f((m_run - m_use) * c2);
+            const float mc = m_use * c2;
+            float psum = 0.f;
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float pv = exp2f(s[nb][r] * c2 - mc);
+                    s[nb][r] = pv;
+                    psum += pv;
+                }
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+#pragma unroll
+            for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
+                bf16x8 pb = pack_bf16x8(s[kb >> 1], (kb & 1) * 8);
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    bf16x8 a = lds_operand_tr(Vs, VS, kb * 16, db * 32, lane);
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
+                }
+            }
+        }
+        have = have_next;
+    }
+
+    // epilogue: normalise, optional merge with the partial result already in (o, lse)
+    const float l_tot = xhalf_sum(l_run);
+    float lse_new = (l_tot > 0.f) ? m_run * p.scale + logf(l_tot) : -INFINITY;
+    float w_cur = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    float w_old = 0.f;
+    float *lse_p = p.lse + ((long long)b * p.Hq + h) * p.Sq + my_row;
+    if ((p.flags & LTR_MERGE) && row_ok) {
+        const float lse_old = *lse_p;
+        const float mxl = fmaxf(lse_old, lse_new);
+        if (mxl == -INFINITY) {
+            w_cur = 0.f;
+        } else {
+            const float e_old = expf(lse_old - mxl), e_new = expf(lse_new - mxl);
+            const float tot = e_old + e_new;
+            w_old = e_old / tot;
+            w_cur *= e_new / tot;
+            lse_new = mxl + logf(tot);
+        }
+    }
+    if (row_ok) {
+        if (hh == 0) *lse_p = lse_new;
+        const long long ooff = b * p.os[0] + (long long)my_row * p.os[1] + h * p.os[2];
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = db * 32 + 8 * g + 4 * hh;
+                f32x4 val;
+#pragma unroll
+                for (int e = 0; e < 4; e++) val[e] = oacc[db][4 * g + e] * w_cur;
+                if (p.o_f32) {
+                    float *op = (float *)p.o + ooff + d;
+                    if (p.flags & LTR_MERGE) {
+                        f32x4 old = *(const f32x4 *)op;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) val[e] += old[e] * w_old;
+                    }
+                    *(f32x4 *)op = val;
+                } else {
+                    __bf16 *op = (__bf16 *)p.o + ooff + d;
+                    if (p.flags & LTR_MERGE) {
+                        bf16x4 old = *(const bf16x4 *)op;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) val[e] += (float)old[e] * w_old;
+                    }
+                    bf16x4 ob;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) ob[e] = (__bf16)val[e];
+                    *(bf16x4 *)op = ob;
+                }
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------ forward, fp32
+// One lane per query row, 64 rows per block, K/V tiles of 32 keys broadcast from LDS.
+template <int D>
+__global__ __launch_bounds__(64) void fwd_f32_kernel(const FwdParams p) {
+    constexpr int BN = 32;
+    __shared__ __attribute__((aligned(16))) float Ks[BN * D];
+    __shared__ __attribute__((aligned(16))) float Vs[BN * D];
+    const int tid = threadIdx.x;
+    const bool causal = p.flags & LTR_CAUSAL;
+    int idx = blockIdx.x;
+    const int qt = p.n_qtiles - 1 - idx / (p.B * p.Hq);
+    const int bh = idx % (p.B * p.Hq);
+    const int b = bh / p.Hq, h = bh % p.Hq, hkv = h / p.n_rep;
+    const int row0 = qt * 64, my_row = row0 + tid;
+    const bool row_ok = my_row < p.Sq;
+    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int blk_lo, blk_hi;
+    q_pos_range(row0, min(row0 + 64, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+
+    float q[D], o[D];
+    {
+        const float *qp = (const float *)p.q + b * p.qs[0] + (long long)my_row * p.qs[1] + h * p.qs[2];
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            q[d] = row_ok ? qp[d] : 0.f;
+            o[d] = 0.f;
+        }
+    }
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int c = 0; c < p.n_chunks; c++) {
+        const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
+        const int nvis = causal ? max(0, min(sk, blk_hi - pos0 + 1)) : sk;
+        const float *kp = (const float *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+        const float *vp = (const float *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+        for (int key0 = 0; key0 < nvis; key0 += BN) {
+            __syncthreads();
+            for (int i = tid; i < BN * D / 4; i += 64) {
+                int key = key0 + i / (D / 4), dc = i % (D / 4);
+                f32x4 kv = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
+                if (key < sk) {
+                    kv = *(const f32x4 *)(kp + (long long)key * p.ks[1] + dc * 4);
+                    vv = *(const f32x4 *)(vp + (long long)key * p.vs[1] + dc * 4);
+                }
+                *(f32x4 *)(Ks + i * 4) = kv;
+                *(f32x4 *)(Vs + i * 4) = vv;
+            }
+            __syncthreads();
+            float s[BN];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < BN; j++) {
+                float acc = 0.f;
+#pragma unroll
+                for (int d = 0; d < D; d++) acc = fmaf(q[d], Ks[j * D + d], acc);
+                acc *= p.scale;
+                const int key = key0 + j;
+                const bool vis = key < sk && (!causal || pos0 + key <= my_pos);
+                s[j] = vis ? acc : -INFINITY;
+                mx = fmaxf(mx, s[j]);
+            }
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = expf(m_run - m_use);
+            l_run *= alpha;
+#pragma unroll
+            for (int d = 0; d < D; d++) o[d] *= alpha;
+#pragma unroll
+            for (int j = 0; j < BN; j++) {
+                const float pj = expf(s[j] - m_use);
+                l_run += pj;
+#pragma unroll
+                for (int d = 0; d < D; d++) o[d] = fmaf(pj, Vs[j * D + d], o[d]);
+            }
+            m_run = m_new;
+        }
+    }
+    if (!row_ok) return;
+    float lse_new = (l_run > 0.f) ? m_run + logf(l_run) : -INFINITY;
+    float w_cur = (l_run > 0.f) ? 1.f / l_run : 0.f, w_old = 0.f;
+    float *lse_p = p.lse + ((long long)b * p.Hq + h) * p.Sq + my_row;
+    if (p.flags & LTR_MERGE) {
+        const float lse_old = *lse_p;
+        const float mxl = fmaxf(lse_old, lse_new);
+        if (mxl == -INFINITY) {
+            w_cur = 0.f;
+        } else {
+            const float e_old = expf(lse_old - mxl), e_new = expf(lse_new - mxl);
+            const float tot = e_old + e_new;
+            w_old = e_old / tot;
+            w_cur *= e_new / tot;
+            lse_new = mxl + logf(tot);
+        }
+    }
+    *lse_p = lse_new;
+    float *op = (float *)p.o + b * p.os[0] + (long long)my_row * p.os[1] + h * p.os[2];
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        float val = o[d] * w_cur;
+        if (p.flags & LTR_MERGE) val += op[d] * w_old;
+        op[d] = val;
+    }
+}
+
+// ------------------------------------------------------------------------------ delta
+// 16 lanes per (b, h, row); each lane covers D/16 contiguous elements.
+__global__ __launch_bounds__(256) void delta_kernel(const DeltaParams p) {
+    const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long rowid = gid >> 4;
+    const int sub = gid & 15;
+    const long long nrows = (long long)p.B * p.Hq * p.Sq;
+    float acc = 0.f;
+    if (rowid < nrows) {
+        const int i = rowid % p.Sq;
+        const int h = (rowid / p.Sq) % p.Hq;
+        const int b = rowid / ((long long)p.Sq * p.Hq);
+        const long long oo = b * p.os[0] + (long long)i * p.os[1] + h * p.os[2];
+        const long long od = b * p.dos[0] + (long long)i * p.dos[1] + h * p.dos[2];
+        const int per = p.D / 16;
+        for (int e = 0; e < per; e++) {
+            const int d = sub * per + e;
+            const float ov = p.o_f32 ? ((const float *)p.o)[oo + d] : (float)((const __bf16 *)p.o)[oo + d];
+            const float dv = p.do_f32 ? ((const float *)p.d_o)[od + d] : (float)((const __bf16 *)p.d_o)[od + d];
+            acc = fmaf(ov, dv, acc);
+        }
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 16);
+    if (rowid < nrows && sub == 0) p.delta[rowid] = acc;
+}
+
+__global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst, long long n) {
+    long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i + 3 < n) {
+        f32x4 x = *(const f32x4 *)(src + i);
+        bf16x4 y;
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = (__bf16)x[e];
+        *(bf16x4 *)(dst + i) = y;
+    } else {
+        for (; i < n; i++) dst[i] = (__bf16)src[i];
+    }
+}
+
+// ------------------------------------------------------------------------------ backward, bf16
+template <int D>
+__global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
+    constexpr int BN = 128;      // keys per block, 32 per wave
+    constexpr int BM = 32;       // query rows per iteration
+    constexpr int QS = D + 8;    // Q / dO tile row stride (elements)
+    constexpr int DSS = BN + 8;  // dS tile row stride
+    constexpr int CPR = D / 8;
+    constexpr int NLD = BM * CPR / 256;  // 16-byte chunks per thread per tile (2 for D=128, 1 for D=64)
+    static_assert(NLD >= 1, "tile too small");
+    __shared__ __attribute__((aligned(16))) __bf16 Qs[BM * QS];
+    __shared__ __attribute__((aligned(16))) __bf16 dOs[BM * QS];
+    __shared__ __attribute__((aligned(16))) __bf16 dSs[BM * DSS];
+    __shared__ __attribute__((aligned(16))) float lse_s[BM];
+    __shared__ __attribute__((aligned(16))) float dlt_s[BM];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const bool causal = p.flags & LTR_CAUSAL;
+
+    // block -> (batch, kv head, chunk, key tile); same XCD grouping as the forward
+    int idx = blockIdx.x, pair, rest;
+    const int P = p.B * p.Hkv;
+    if ((P & 7) == 0) {
+        int xcd = idx & 7, j = idx >> 3, pp = P >> 3;
+        pair = (j % pp) * 8 + xcd;
+        rest = j / pp;
+    } else {
+        pair = idx % P;
+        rest = idx / P;
+    }
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv;
+    int c = 0, kt = rest;
+    for (; c < p.n_chunks; c++) {
+        int n = (p.chunk[c].sk + BN - 1) / BN;
+        if (kt < n) break;
+        kt -= n;
+    }
+    if (c >= p.n_chunks) return;
+    const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
+    const int key0 = kt * BN;
+    const int my_key = key0 + w * 32 + l32;     // this lane's key in S / dP / dK^T / dV^T tiles
+    const bool key_ok = my_key < sk;
+    const int my_kpos = pos0 + my_key;
+    const int tile_kpos_lo = pos0 + key0;
+    const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
+
+    // resident operands.  kreg / vreg: B operand of S = Q K^T and dP = dO V^T, lane (key l32,
+    // half hh) holds d = 16*kb + 8*hh .. +7.  ktreg: B operand of dQ = dS K over this wave's
+    // 32 columns of D (d = 32*w + l32) and all 128 keys: K-dim values are keys 16*kb + 8*hh + e.
+    bf16x8 kreg[D / 16], vreg[D / 16], ktreg[BN / 16];
+    {
+        const __bf16 *kp = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+        const __bf16 *vp = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) {
+            uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0);
+            if (key_ok) {
+                kx = *(const uint4 *)(kp + (long long)my_key * p.ks[1] + kb * 16 + 8 * hh);
+                vx = *(const uint4 *)(vp + (long long)my_key * p.vs[1] + kb * 16 + 8 * hh);
+            }
+            kreg[kb] = as_bf16x8(kx);
+            vreg[kb] = as_bf16x8(vx);
+        }
+        const int dcol = (w * 32 + l32) % D;  // D = 64: waves 2,3 repeat columns 0..63 (results unused)
+#pragma unroll
+        for (int kb = 0; kb < BN / 16; kb++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                int key = key0 + kb * 16 + 8 * hh + e;
+                ktreg[kb][e] = key < sk ? kp[(long long)key * p.ks[1] + dcol] : (__bf16)0.f;
+            }
+        }
+    }
+
+    f32x16 dkacc[D / 32], dvacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            dkacc[i][r] = 0.f;
+            dvacc[i][r] = 0.f;
+        }
+    const float c2 = p.scale * LTR_LOG2E;
+
+    for (int rep = 0; rep < p.n_rep; rep++) {
+        const int h = hkv * p.n_rep + rep;
+        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
+        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
+        const float *lsep = p.lse + ((long long)b * p.Hq + h) * p.Sq;
+        const float *dltp = p.delta + ((long long)b * p.Hq + h) * p.Sq;
+        float *dqp = p.dq + b * p.dqs[0] + h * p.dqs[2];
+        for (int qt = 0; qt < p.n_qtiles; qt++) {
+            const int row0 = qt * BM;
+            int t_lo, t_hi;
+            q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], t_lo, t_hi);
+            if (causal && t_hi < tile_kpos_lo) continue;  // no query of the tile sees any key of the block
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                int id = tid + 256 * i;
+                int r = id / CPR, dc = id % CPR;
+                uint4 qx = make_uint4(0, 0, 0, 0), dx = make_uint4(0, 0, 0, 0);
+                if (row0 + r < p.Sq) {
+                    qx = *(const uint4 *)(qp + (long long)(row0 + r) * p.qs[1] + dc * 8);
+                    dx = *(const uint4 *)(dop + (long long)(row0 + r) * p.dos[1] + dc * 8);
+                }
+                *(uint4 *)(Qs + r * QS + dc * 8) = qx;
+                *(uint4 *)(dOs + r * QS + dc * 8) = dx;
+            }
+            if (tid < BM) {
+                lse_s[tid] = (row0 + tid < p.Sq) ? lsep[row0 + tid] : INFINITY;
+            } else if (tid < 2 * BM) {
+                dlt_s[tid - BM] = (row0 + tid - BM < p.Sq) ? dltp[row0 + tid - BM] : 0.f;
+            }
+            __syncthreads();
+
+            // wave-uniform skip: none of this wave's keys is visible to any row of the tile
+            const bool wave_active = !causal || (pos0 + key0 + w * 32 <= t_hi);
+            f32x16 s, dp;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                s[r] = 0.f;
+                dp[r] = 0.f;
+            }
+            if (wave_active) {
+#pragma unroll
+                for (int kb = 0; kb < D / 16; kb++) {
+                    bf16x8 a = *(const bf16x8 *)(Qs + l32 * QS + kb * 16 + 8 * hh);
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kreg[kb], s, 0, 0, 0);
+                }
+#pragma unroll
+                for (int kb = 0; kb < D / 16; kb++) {
+                    bf16x8 a = *(const bf16x8 *)(dOs + l32 * QS + kb * 16 + 8 * hh);
+                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vreg[kb], dp, 0, 0, 0);
+                }
+                const bool need_mask = (key0 + BN > sk) || (causal && tile_kpos_hi > t_lo);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 lv = *(const f32x4 *)(lse_s + 8 * g + 4 * hh);
+                    const f32x4 dv = *(const f32x4 *)(dlt_s + 8 * g + 4 * hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int r = 4 * g + e;
+                        float pv = exp2f(s[r] * c2 - lv[e] * LTR_LOG2E);
+                        if (need_mask) {
+                            const int qrow = row0 + 8 * g + 4 * hh + e;
+                            const int qpos = q_position(qrow, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+                            const bool vis = key_ok && (!causal || my_kpos <= qpos);
+                            pv = vis ? pv : 0.f;
+                        }
+                        s[r] = pv;
+                        dp[r] = pv * (dp[r] - dv[e]);
+                    }
+                }
+                // dV^T += dO^T P and dK^T += Q^T dS: contraction over the 32 query rows
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    bf16x8 pb = pack_bf16x8(s, kb * 8);
+                    bf16x8 dsb = pack_bf16x8(dp, kb * 8);
+#pragma unroll
+                    for (int db = 0; db < D / 32; db++) {
+                        bf16x8 a = lds_operand_tr(dOs, QS, kb * 16, db * 32, lane);
+                        dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, dvacc[db], 0, 0, 0);
+                        bf16x8 a2 = lds_operand_tr(Qs, QS, kb * 16, db * 32, lane);
+                        dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, dsb, dkacc[db], 0, 0, 0);
+                    }
+                }
+            }
+            // dS tile [query][key] to LDS (zeros from inactive waves)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int qi = 8 * (r / 4) + 4 * hh + (r % 4);
+                dSs[qi * DSS + w * 32 + l32] = (__bf16)dp[r];
+            }
+            __syncthreads();
+            // dQ[:, 32w .. 32w+31] = dS (32 x 128 keys) K[:, 32w ..]
+            if (w * 32 < D) {
+                f32x16 dq;
+#pragma unroll
+                for (int r = 0; r < 16; r++) dq[r] = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < BN / 16; kb++) {
+                    bf16x8 a = *(const bf16x8 *)(dSs + l32 * DSS + kb * 16 + 8 * hh);
+                    dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, ktreg[kb], dq, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int qrow = row0 + 8 * (r / 4) + 4 * hh + (r % 4);
+                    if (qrow < p.Sq) atomicAdd(dqp + (long long)qrow * p.dqs[1] + w * 32 + l32, dq[r] * p.scale);
+                }
+            }
+        }
+    }
+
+    // dK^T / dV^T tiles: lane (key l32 of this wave, half hh), register r -> d = 32*db + 8*(r/4) + 4hh + r%4
+    if (key_ok) {
+        float *dkp = p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2];
+        float *dvp = p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2];
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = db * 32 + 8 * g + 4 * hh;
+                f32x4 ok = *(const f32x4 *)(dkp + d), ov = *(const f32x4 *)(dvp + d);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    ok[e] += dkacc[db][4 * g + e] * p.scale;
+                    ov[e] += dvacc[db][4 * g + e];
+                }
+                *(f32x4 *)(dkp + d) = ok;
+                *(f32x4 *)(dvp + d) = ov;
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------ host side
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+int check_device() {
+    // gfx950 only; the answer is cached per process (read-only after first use)
+    static int cached = 0;  // 0 unknown, 1 ok, -1 bad
+    if (cached == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_EDEVICE;
+        const char *a = prop.gcnArchName;
+        cached = (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') ? 1 : -1;
+    }
+    return cached == 1 ? LTR_OK : LTR_EDEVICE;
+}
+
+bool strides_ok(const int64_t *s, int elem_bytes) {
+    const int per16 = 16 / elem_bytes;
+    for (int i = 0; i < 3; i++)
+        if (s[i] < 0 || (s[i] % per16) != 0) return false;
+    return true;
+}
+
+int fits_i32(int64_t x) { return x >= 0 && x < (int64_t)0x7fffffff; }
+
+}  // namespace
+
+extern "C" int ltr_abi_version(void) { return LTR_ABI_VERSION; }
+
+extern "C" const char *ltr_strerror(int code) {
+    switch (code) {
+        case LTR_OK: return "ok";
+        case LTR_EINVAL: return "invalid argument (null pointer, bad size or flag)";
+        case LTR_EUNSUP: return "unsupported head dim / dtype combination";
+        case LTR_EALIGN: return "pointer or stride not 16-byte aligned";
+        case LTR_ELAUNCH: return "HIP launch error";
+        case LTR_EDEVICE: return "current device is not gfx950";
+        default: return "unknown error";
+    }
+}
+
+extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
+    if (!a || !a->q || !a->o || !a->lse) return LTR_EINVAL;
+    if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
+    if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE)) return LTR_EINVAL;
+    if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
+    if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
+    if (a->o_dtype != LTR_BF16 && a->o_dtype != LTR_F32) return LTR_EUNSUP;
+    if (a->io_dtype == LTR_F32 && a->o_dtype != LTR_F32) return LTR_EUNSUP;
+    if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
+    if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
+    const int eb = a->io_dtype == LTR_BF16 ? 2 : 4, ob = a->o_dtype == LTR_BF16 ? 2 : 4;
+    if (!aligned16(a->q) || !aligned16(a->o) || !aligned16(a->lse)) return LTR_EALIGN;
+    if (!strides_ok(a->q_stride, eb) || !strides_ok(a->k_stride, eb) || !strides_ok(a->v_stride, eb)) return LTR_EALIGN;
+    // o rows are written in 4-element groups
+    for (int i = 0; i < 3; i++)
+        if (a->o_stride[i] < 0 || (a->o_stride[i] * ob) % 8) return LTR_EALIGN;
+    FwdParams p;
+    for (int c = 0; c < a->n_chunks; c++) {
+        const ltr_kv_chunk &ch = a->chunk[c];
+        if (!ch.k || !ch.v || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
+        if (!aligned16(ch.k) || !aligned16(ch.v)) return LTR_EALIGN;
+        p.chunk[c].k = ch.k;
+        p.chunk[c].v = ch.v;
+        p.chunk[c].dk = nullptr;
+        p.chunk[c].dv = nullptr;
+        p.chunk[c].sk = (int)ch.sk;
+        p.chunk[c].pos0 = (int)ch.pos0;
+    }
+    int rc = check_device();
+    if (rc) return rc;
+    p.q = a->q;
+    p.o = a->o;
+    p.lse = a->lse;
+    p.B = a->B;
+    p.Hq = a->Hq;
+    p.Hkv = a->Hkv;
+    p.n_rep = a->Hq / a->Hkv;
+    p.Sq = (int)a->Sq;
+    for (int i = 0; i < 3; i++) {
+        p.qs[i] = a->q_stride[i];
+        p.os[i] = a->o_stride[i];
+        p.ks[i] = a->k_stride[i];
+        p.vs[i] = a->v_stride[i];
+    }
+    p.q_pos0[0] = (int)a->q_pos0[0];
+    p.q_pos0[1] = (int)a->q_pos0[1];
+    p.q_split = (int)a->q_split;
+    p.scale = a->scale;
+    p.flags = a->flags;
+    p.o_f32 = a->o_dtype == LTR_F32;
+    p.n_chunks = a->n_chunks;
+    hipStream_t st = (hipStream_t)stream;
+    if (a->io_dtype == LTR_BF16) {
+        p.n_qtiles = (p.Sq + 127) / 128;
+        const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
+        if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+        if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), 0, st, p);
+    } else {
+        p.n_qtiles = (p.Sq + 63) / 64;
+        const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
+        if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+        if (a->D == 128) hipLaunchKernelGGL(fwd_f32_kernel<128>, dim3((unsigned)nblk), dim3(64), 0, st, p);
+        else hipLaunchKernelGGL(fwd_f32_kernel<64>, dim3((unsigned)nblk), dim3(64), 0, st, p);
+    }
+    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+}
+
+extern "C" int ltr_attn_bwd_delta(const ltr_attn_delta_args *a, void *stream) {
+    if (!a || !a->o || !a->d_o || !a->delta) return LTR_EINVAL;
+    if (a->B <= 0 || a->Hq <= 0 || a->Sq <= 0 || !fits_i32(a->Sq)) return LTR_EINVAL;
+    if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
+    if ((a->o_dtype != LTR_BF16 && a->o_dtype != LTR_F32) || (a->do_dtype != LTR_BF16 && a->do_dtype != LTR_F32))
+        return LTR_EUNSUP;
+    for (int i = 0; i < 3; i++)
+        if (a->o_stride[i] < 0 || a->do_stride[i] < 0) return LTR_EINVAL;
+    int rc = check_device();
+    if (rc) return rc;
+    DeltaParams p;
+    p.o = a->o;
+    p.d_o = a->d_o;
+    p.delta = a->delta;
+    p.B = a->B;
+    p.Hq = a->Hq;
+    p.D = a->D;
+    p.Sq = (int)a->Sq;
+    for (int i = 0; i < 3; i++) {
+        p.os[i] = a->o_stride[i];
+        p.dos[i] = a->do_stride[i];
+    }
+    p.o_f32 = a->o_dtype == LTR_F32;
+    p.do_f32 = a->do_dtype == LTR_F32;
+    const long long nthreads = (long long)p.B * p.Hq * p.Sq * 16;
+    const long long nblk = (nthreads + 255) / 256;
+    if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+    hipLaunchKernelGGL(delta_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream, p);
+    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+}
+
+extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
+    if (!a || !a->q || !a->d_o || !a->lse || !a->delta || !a->dq) return LTR_EINVAL;
+    if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
+    if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
+    if (a->flags & ~LTR_CAUSAL) return LTR_EINVAL;
+    if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
+    if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;
+    if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
+    if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
+    if (!aligned16(a->q) || !aligned16(a->d_o) || !aligned16(a->dq)) return LTR_EALIGN;
+    if (!strides_ok(a->q_stride, 2) || !strides_ok(a->do_stride, 2) || !strides_ok(a->k_stride, 2) ||
+        !strides_ok(a->v_stride, 2) || !strides_ok(a->dk_stride, 4) || !strides_ok(a->dv_stride, 4))
+        return LTR_EALIGN;
+    for (int i = 0; i < 3; i++)
+        if (a->dq_stride[i] < 0) return LTR_EINVAL;
+    BwdParams p;
+    long long tiles = 0;
+    for (int c = 0; c < a->n_chunks; c++) {
+        const ltr_kv_chunk &ch = a->chunk[c];
+        if (!ch.k || !ch.v || !ch.dk || !ch.dv || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk))
+            return LTR_EINVAL;
+        if (!aligned16(ch.k) || !aligned16(ch.v) || !aligned16(ch.dk) || !aligned16(ch.dv)) return LTR_EALIGN;
+        p.chunk[c].k = ch.k;
+        p.chunk[c].v = ch.v;
+        p.chunk[c].dk = (float *)ch.dk;
+        p.chunk[c].dv = (float *)ch.dv;
+        p.chunk[c].sk = (int)ch.sk;
+        p.chunk[c].pos0 = (int)ch.pos0;
+        tiles += (ch.sk + 127) / 128;
+    }
+    int rc = check_device();
+    if (rc) return rc;
+    p.q = a->q;
+    p.d_o = a->d_o;
+    p.lse = a->lse;
+    p.delta = a->delta;
+    p.dq = a->dq;
+    p.B = a->B;
+    p.Hq = a->Hq;
+    p.Hkv = a->Hkv;
+    p.n_rep = a->Hq / a->Hkv;
+    p.Sq = (int)a->Sq;
+    p.n_qtiles = (p.Sq + 31) / 32;
+    for (int i = 0; i < 3; i++) {
+        p.qs[i] = a->q_stride[i];
+        p.dos[i] = a->do_stride[i];
+        p.dqs[i] = a->dq_stride[i];
+        p.ks[i] = a->k_stride[i];
+        p.vs[i] = a->v_stride[i];
+        p.dks[i] = a->dk_stride[i];
+        p.dvs[i] = a->dv_stride[i];
+    }
+    p.q_pos0[0] = (int)a->q_pos0[0];
+    p.q_pos0[1] = (int)a->q_pos0[1];
+    p.q_split = (int)a->q_split;
+    p.scale = a->scale;
+    p.flags = a->flags;
+    p.n_chunks = a->n_chunks;
+    p.tiles_total = (int)tiles;
+    const long long nblk = tiles * p.B * p.Hkv;
+    if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+    hipStream_t st = (hipStream_t)stream;
+    if (a->D == 128) hipLaunchKernelGGL(bwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(bwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), 0, st, p);
+    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+}
+
+extern "C" int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream) {
+    if (!src || !dst || n < 0) return LTR_EINVAL;
+    if (n == 0) return LTR_OK;
+    if (!aligned16(src) || ((uintptr_t)dst & 7)) return LTR_EALIGN;
+    int rc = check_device();
+    if (rc) return rc;
+    const long long nblk = (n / 4 + 256) / 256;
+    if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+    hipLaunchKernelGGL(cast_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream, src, (__bf16 *)dst,
+                       (long long)n);
+    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+}

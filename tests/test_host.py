@@ -1,0 +1,140 @@
+"""CPU tests of the host side: the C-ABI library loads and exports what include/ltr_attn.h
+declares, argument validation answers without a GPU, and the Ulysses permutation matches the
+oracle's restatement of parallel_cp.py:49-96."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import ring_attention_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib():
+    from lightron_amd import _lib as L
+    if not os.path.exists(L.LIB_PATH):
+        import lightron_amd.build as b
+        b.build()
+    return L, L.load()
+
+
+def test_header_symbols_exported():
+    L, lib = _lib()
+    hdr = open(os.path.join(ROOT, "include", "ltr_attn.h")).read()
+    declared = set(re.findall(r"^(?:int|const char \*)\s*\*?(ltr_\w+)\(", hdr, flags=re.M))
+    assert declared == set(L.EXPORTS), declared
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.ltr_abi_version() == 1
+    assert lib.ltr_strerror(0) == b"ok" and b"aligned" in lib.ltr_strerror(-3)
+
+
+def test_struct_layout_matches_header():
+    # sizes computed from the header's field lists: catches a drifted ctypes mirror
+    L, _ = _lib()
+    assert ctypes.sizeof(L.KvChunk) == 48
+    assert ctypes.sizeof(L.FwdArgs) == 3 * 8 + 4 * 4 + 8 + 4 * 24 + 16 + 8 + 4 * 5 + 4 + 32 * 48
+    assert ctypes.sizeof(L.DeltaArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
+    assert ctypes.sizeof(L.BwdArgs) == 5 * 8 + 4 * 4 + 8 + 7 * 24 + 16 + 8 + 4 * 4 + 32 * 48
+
+
+def test_validation_without_gpu():
+    L, lib = _lib()
+    assert lib.ltr_attn_fwd(None, None) == -1
+    a = L.FwdArgs()
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -1            # null pointers
+    a.q = a.o = a.lse = 4096
+    a.B, a.Hq, a.Hkv, a.D, a.Sq, a.n_chunks = 1, 4, 3, 128, 16, 1
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -1            # Hq % Hkv
+    a.Hkv, a.D = 2, 96
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -2            # head dim
+    a.D, a.n_chunks = 128, 33
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -1            # too many chunks
+    a.n_chunks, a.q, a.q_split = 1, 4100, 16
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -3            # misaligned q
+    a.q = 4096
+    a.q_stride[1] = 4                                               # 8-byte row stride in bf16
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -3
+    assert lib.ltr_attn_bwd(None, None) == -1 and lib.ltr_attn_bwd_delta(None, None) == -1
+    assert lib.ltr_cast_f32_to_bf16(None, None, 4, None) == -1
+    assert lib.ltr_cast_f32_to_bf16(4096, 4096, 0, None) == 0       # empty input is a no-op
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from lightron_amd import _lib as L
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libltr_attn.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        L.load()
+
+
+def test_cpu_tensors_are_refused():
+    import lightron_amd as la
+    q = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        la.attn_fwd(q, [q], [q], [0])
+
+
+@pytest.mark.parametrize("W", [1, 2, 4])
+def test_seq_all_to_all_matches_oracle_and_backward(W):
+    import lightron_amd as la
+    B, Sl, H, D = 2, 3, 8, 4
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(W, B, Sl, H, D, generator=g, requires_grad=True)
+    grp = la.LocalCPGroup(W)
+    y = la._all_to_all(x if W > 1 else x[0], 2, 1, grp)
+    ref = orc.seq_all_to_all([x[r].detach() for r in range(W)], 2, 1)
+    if W == 1:
+        assert y is x[0] or torch.equal(y, x[0])
+        return
+    for r in range(W):
+        assert torch.equal(y[r], ref[r])
+    back = la._all_to_all(y, 1, 2, grp)
+    assert torch.equal(back, x)
+    # backward = the exchange with the two dims swapped (parallel_cp.py:85-93)
+    gy = torch.randn(y.shape, generator=g)
+    y.backward(gy)
+    gref = orc.seq_all_to_all([gy[r] for r in range(W)], 1, 2)
+    for r in range(W):
+        assert torch.equal(x.grad[r], gref[r])
+
+
+def test_seq_all_to_all_refuses_indivisible_and_real_groups():
+    import lightron_amd as la
+    x = torch.zeros(4, 1, 2, 6, 2)
+    with pytest.raises(AssertionError):
+        la._all_to_all(x, 2, 1, la.LocalCPGroup(4))
+    assert torch.equal(la._all_to_all(x, 2, 1, None), x)
+    with pytest.raises(NotImplementedError):
+        la._all_to_all(x, 2, 1, object())
+
+
+def test_ring_descriptor_order_and_positions():
+    from lightron_amd.ring_attention import LocalRing, _chunk_table
+    ring = LocalRing(2, 4, kv=[(torch.zeros(1, 8, 1, 4), torch.zeros(1, 8, 1, 4))] * 4, layout="zigzag")
+    assert ring.order() == orc.ring_order(2, 4) == [2, 1, 0, 3]
+    ks, vs, pos = _chunk_table(ring, None, None, 8)
+    exp = []
+    for j in ring.order():
+        p = orc.zigzag_positions(j, 4, 32)
+        exp += [int(p[0]), int(p[4])]
+    assert pos == exp and all(k.shape[1] == 4 for k in ks)
+    with pytest.raises(NotImplementedError):
+        import lightron_amd as la
+        la.ring_attention_kernel(torch.zeros(1, 8, 1, 64), None, None, object(), None)
+
+
+def test_rope_helpers_match_oracle():
+    import lightron_amd as la
+    fc = la.precompute_freqs_cis(16, 32)
+    assert (fc - orc.precompute_freqs_cis(16, 32)).abs().max() < 1e-6
+    g = torch.Generator().manual_seed(5)
+    q, k = torch.randn(2, 32, 3, 16, generator=g), torch.randn(2, 32, 3, 16, generator=g)
+    a, b = la.apply_rotary_emb(q, k, fc)
+    c, d = orc.apply_rotary_emb(q, k, fc)
+    assert (a - c).abs().max() < 1e-6 and (b - d).abs().max() < 1e-6
+    with pytest.raises(AssertionError):
+        la.apply_rotary_emb(q, k, fc[:16])
