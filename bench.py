@@ -1,0 +1,238 @@
+"""Benchmark of the ring-attention hot path on one MI355X.
+
+Default workload (the one the headline metric is quoted on): B=1, Hq=32, Hkv=8, D=128,
+S=32768, bf16, causal, zig-zag assignment over 8 ranks; one "step" runs every rank's share
+(forward over the 16 half-chunk KV table, DELTA, recompute backward with dK/dV accumulated
+in fp32 across shares, final casts) so a step is the whole sequence's forward+backward.
+Inputs are synthetic N(0,1) (seed 0) and resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is causal-adjusted TFLOP/s: 14*B*Hq*D*N_pairs flops (2 GEMMs
+forward, 5 backward, unmasked pairs only) divided by the step time.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
+
+
+def _workload(name):
+    # (B, Hq, Hkv, D, S_total, W ranks, layout, causal, ranks to run, bwd)
+    if name == "c3":
+        return dict(B=1, Hq=32, Hkv=8, D=128, S=32768, W=8, layout="zigzag", causal=True,
+                    ranks=list(range(8)), bwd=True,
+                    desc="config 3: GQA 32/8 D=128 S=32768 bf16 causal, 8 zig-zag rank shares, fwd+bwd")
+    if name == "c2":
+        return dict(B=4, Hq=32, Hkv=32, D=128, S=8192, W=8, layout="contiguous", causal=True,
+                    ranks=[7], bwd=False,
+                    desc="config 2: B=4 H=32 D=128, last rank's Q chunk 1024 vs 8x1024 KV, bf16 causal, fwd")
+    if name == "c4":
+        return dict(B=1, Hq=8, Hkv=8, D=128, S=131072, W=16, layout="contiguous", causal=True,
+                    ranks=[15], bwd=True,
+                    desc="config 4: H=8 D=128 S=131072, rank 15's 8192-token Q chunk vs 16x8192 KV, fwd+bwd")
+    if name == "c5":
+        return dict(B=8, Hq=4, Hkv=4, D=64, S=4096, W=1, layout="contiguous", causal=False,
+                    ranks=[0], bwd=True,
+                    desc="config 5: B=8, 4 local heads of 16, D=64, S=4096, non-causal, fwd+bwd")
+    raise SystemExit("unknown workload %r" % name)
+
+
+def _rank_positions(cfg, r):
+    import torch
+    W, S = cfg["W"], cfg["S"]
+    if cfg["layout"] == "zigzag":
+        hc = S // (2 * W)
+        return torch.cat([torch.arange(r * hc, (r + 1) * hc), torch.arange((2 * W - 1 - r) * hc, (2 * W - r) * hc)])
+    sl = S // W
+    return torch.arange(r * sl, (r + 1) * sl)
+
+
+def _n_pairs(cfg, r):
+    import torch
+    qp = _rank_positions(cfg, r)
+    if not cfg["causal"]:
+        return qp.numel() * cfg["S"]
+    return int((qp + 1).sum())          # keys 0..pos visible
+
+
+def _cpu_baseline(cfg, threads):
+    """The oracle (the reference composition restated in torch) timed on the host cores on a
+    bounded sample: one off-diagonal and one diagonal 2048x2048 block-step of the workload's
+    head configuration, forward by the online-softmax recurrence and backward by autograd
+    through it, fp32."""
+    import torch
+    from oracle import ring_attention_oracle as orc
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    blk = min(2048, cfg["S"])
+    B, Hq, Hkv, D = cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["D"]
+    q = torch.randn(B, blk, Hq, D, generator=g).requires_grad_(True)
+    k = torch.randn(B, blk, Hkv, D, generator=g).requires_grad_(True)
+    v = torch.randn(B, blk, Hkv, D, generator=g).requires_grad_(True)
+    do = torch.randn(B, blk, Hq, D, generator=g)
+    pos = torch.arange(blk)
+    flops = 0.0
+    t_total = 0.0
+    reps = 0
+    cases = [(pos + blk, False), (pos, True)] if cfg["causal"] else [(pos, False)]
+    t_start = time.time()
+    while t_total < 10.0 and time.time() - t_start < 40.0:
+        for qpos, diag in cases:
+            t0 = time.time()
+            o, _ = orc.ring_attention_recurrence(q, [(k, v)], qpos, [pos], cfg["causal"])
+            if cfg["bwd"]:
+                o.backward(do)
+            t_total += time.time() - t0
+            pairs = blk * (blk + 1) // 2 if diag else blk * blk
+            flops += (14.0 if cfg["bwd"] else 4.0) * B * Hq * D * pairs
+        reps += 1
+    return {"value": flops / t_total / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%d x (%s) %dx%d block-steps, B=%d Hq=%d Hkv=%d D=%d, fp32 torch CPU, %s; %.1f s" % (
+                reps, "off-diagonal + diagonal" if cfg["causal"] else "full", blk, blk, B, Hq, Hkv, D,
+                "fwd + autograd bwd" if cfg["bwd"] else "fwd", t_total)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (no collectives, no sharding across GPUs); "
+                         "run with --gpus 1")
+    import torch
+    import lightron_amd as la
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    la._lib.load()
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    cfg = _workload(args.workload)
+    B, Hq, Hkv, D, S, W = (cfg[x] for x in ("B", "Hq", "Hkv", "D", "S", "W"))
+    causal, bwd = cfg["causal"], cfg["bwd"]
+    sl = S // W
+
+    # synthetic inputs, generated on the CPU in the order q, k, v, dO, stored rank-major [W, B, S_l, H, D]
+    g = torch.Generator().manual_seed(0)
+    def mk(h):
+        full = torch.randn(B, S, h, D, generator=g).to(torch.bfloat16)
+        return torch.stack([full[:, _rank_positions(cfg, r)] for r in range(W)], 0).to(dev)
+    q_all, k_all, v_all = mk(Hq), mk(Hkv), mk(Hkv)
+    do_all = mk(Hq) if bwd else None
+
+    # per-rank chunk tables in the reference's visiting order
+    tables = {}
+    for r in cfg["ranks"]:
+        ks, vs, dks, dvs, pos = [], [], [], [], []
+        for j in [(r - s) % W for s in range(W)]:
+            if cfg["layout"] == "zigzag":
+                hc = sl // 2
+                for half, p0 in ((slice(0, hc), j * hc), (slice(hc, sl), (2 * W - 1 - j) * hc)):
+                    ks.append(k_all[j][:, half]); vs.append(v_all[j][:, half]); pos.append(p0)
+            else:
+                ks.append(k_all[j]); vs.append(v_all[j]); pos.append(j * sl)
+        if cfg["layout"] == "zigzag":
+            qp, qsplit = (r * (sl // 2), (2 * W - 1 - r) * (sl // 2)), sl // 2
+        else:
+            qp, qsplit = (r * sl, r * sl), sl
+        tables[r] = (ks, vs, pos, qp, qsplit)
+
+    o_all = torch.empty_like(q_all)
+    lse_all = torch.empty(W, B, Hq, sl, dtype=torch.float32, device=dev)
+    if bwd:
+        dq_acc = torch.empty(q_all.shape, dtype=torch.float32, device=dev)
+        dk_acc = torch.empty(k_all.shape, dtype=torch.float32, device=dev)
+        dv_acc = torch.empty(v_all.shape, dtype=torch.float32, device=dev)
+
+    def acc_views(r, acc):
+        out = []
+        for j in [(r - s) % W for s in range(W)]:
+            if cfg["layout"] == "zigzag":
+                hc = sl // 2
+                out += [acc[j][:, :hc], acc[j][:, hc:]]
+            else:
+                out.append(acc[j])
+        return out
+
+    ev = {"fwd": [], "bwd": []}
+
+    def step(timed):
+        if bwd:
+            dq_acc.zero_(); dk_acc.zero_(); dv_acc.zero_()
+        for r in cfg["ranks"]:
+            ks, vs, pos, qp, qsplit = tables[r]
+            if timed:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            la.attn_fwd(q_all[r], ks, vs, pos, qp, qsplit, causal, out=o_all[r], lse=lse_all[r])
+            if timed:
+                e1.record(); ev["fwd"].append((e0, e1))
+            if bwd:
+                delta = la.attn_delta(o_all[r], do_all[r])
+                if timed:
+                    e2, e3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e2.record()
+                la.attn_bwd_accumulate(q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_acc[r],
+                                       acc_views(r, dk_acc), acc_views(r, dv_acc), qp, qsplit, causal)
+                if timed:
+                    e3.record(); ev["bwd"].append((e2, e3))
+        if bwd:
+            la.cast_to_bf16(dq_acc); la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    pairs = sum(_n_pairs(cfg, r) for r in cfg["ranks"])
+    f_fwd = 4.0 * B * Hq * D * pairs
+    f_total = f_fwd * (3.5 if bwd else 1.0)
+    tflops = f_total / dt / 1e12
+    fwd_ms = sum(a.elapsed_time(b) for a, b in ev["fwd"]) / len(ev["fwd"])
+    launches = len(cfg["ranks"])
+    if bwd:
+        bwd_ms = sum(a.elapsed_time(b) for a, b in ev["bwd"]) / len(ev["bwd"])
+        dom, dom_ms, dom_flops = "bwd_bf16_kernel<%d>" % D, bwd_ms, 2.5 * f_fwd / launches
+    else:
+        bwd_ms = None
+        dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_fwd / launches
+    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
+    prop = torch.cuda.get_device_properties(0)
+    out = {
+        "metric": "ring-attn fwd+bwd causal TFLOP/s at S=32k bf16, 1 GPU; % of MFMA peak",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": cfg["desc"], "B": B, "Hq": Hq, "Hkv": Hkv, "D": D, "S": S, "ranks": launches,
+                   "layout": cfg["layout"], "causal": causal, "flops_per_step": f_total},
+        "frac_of_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        "kernels": {"fwd_ms_per_launch": round(fwd_ms, 4),
+                    "fwd_tflops": round(f_fwd / launches / (fwd_ms * 1e-3) / 1e12, 2),
+                    "bwd_ms_per_launch": None if bwd_ms is None else round(bwd_ms, 4),
+                    "bwd_tflops": None if bwd_ms is None else round(2.5 * f_fwd / launches / (bwd_ms * 1e-3) / 1e12, 2)},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None},
+        "device": {"name": prop.name, "cus": prop.multi_processor_count,
+                   "clock_mhz": getattr(prop, "clock_rate", 0) // 1000},
+    }
+    if not args.no_cpu_baseline:
+        threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        out["cpu_baseline"] = _cpu_baseline(cfg, threads)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
