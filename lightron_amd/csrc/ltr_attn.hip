@@ -159,7 +159,7 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16 &s, int base) {
 
 // ------------------------------------------------------------------------------ forward, bf16
 template <int D>
-__global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdParams p) {
+__global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     constexpr int BM = 128, BN = 64;
     constexpr int KS = D + 8;    // K tile row stride (elements): natural 128-bit operand reads
     constexpr int VS = D + 16;   // V tile row stride: transpose reads
@@ -538,22 +538,95 @@ __global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst
 }
 
 // ------------------------------------------------------------------------------ backward, bf16
+// LDS (dynamic): two buffers of {Q tile, dO tile, LSE*log2e, DELTA} for 64 query rows, two dS tiles.
+template <int D>
+struct BwdLds {
+    static constexpr int BN = 128;      // keys per block, 32 per wave
+    static constexpr int BM = 64;       // query rows per iteration (two 32-row MFMA sub-tiles)
+    static constexpr int QS = D + 8;    // Q / dO tile row stride (elements)
+    static constexpr int DSS = BN + 8;  // dS tile row stride
+    static constexpr int TILE = BM * QS;                                 // elements
+    static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, lse, delta
+    static constexpr int DS_BYTES = BM * DSS * 2;
+    static constexpr int TOTAL = 2 * BUF_BYTES + 2 * DS_BYTES;
+};
+
+// One 32-row sub-tile of the backward for one wave (its 32 keys): S and dP by MFMA, P and dS in
+// registers, dV^T / dK^T accumulation, dS written to LDS as [query][key].  Straight-line code
+// around the accumulators: the mask (diagonal and edge tiles only) is a fix-up of P and dS under
+// a wave-uniform branch, so dkacc / dvacc never cross a control-flow merge.
+template <int D>
+__device__ __forceinline__ void bwd_sub_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
+                                             __bf16 *dSs, const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16],
+                                             f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &zero16,
+                                             int r0, int lane, int l32, int hh, int wkey, float c2, bool need_mask,
+                                             bool key_ok, bool causal, int my_kpos, int row_base, int Sq, int q_split,
+                                             int p0, int p1) {
+    constexpr int QS = BwdLds<D>::QS, DSS = BwdLds<D>::DSS;
+    f32x16 s = zero16, dp = zero16;
+#pragma unroll
+    for (int kb = 0; kb < D / 16; kb++) {
+        bf16x8 a = *(const bf16x8 *)(Qs + (r0 + l32) * QS + kb * 16 + 8 * hh);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kreg[kb], s, 0, 0, 0);
+    }
+#pragma unroll
+    for (int kb = 0; kb < D / 16; kb++) {
+        bf16x8 a = *(const bf16x8 *)(dOs + (r0 + l32) * QS + kb * 16 + 8 * hh);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vreg[kb], dp, 0, 0, 0);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const f32x4 lv = *(const f32x4 *)(lse_s + r0 + 8 * g + 4 * hh);
+        const f32x4 dv = *(const f32x4 *)(dlt_s + r0 + 8 * g + 4 * hh);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int r = 4 * g + e;
+            const float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lv[e]);
+            s[r] = pv;
+            dp[r] = pv * (dp[r] - dv[e]);
+        }
+    }
+    if (need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int qrow = row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
+            const int qpos = q_position(qrow, q_split, p0, p1);
+            const bool vis = key_ok && qrow < Sq && (!causal || my_kpos <= qpos);
+            s[r] = vis ? s[r] : 0.f;
+            dp[r] = vis ? dp[r] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+        bf16x8 pb = pack_bf16x8(s, kb * 8);
+        bf16x8 dsb = pack_bf16x8(dp, kb * 8);
+#pragma unroll
+        for (int db = 0; db < D / 32; db++) {
+            bf16x8 a = lds_operand_tr(dOs, QS, r0 + kb * 16, db * 32, lane);
+            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, dvacc[db], 0, 0, 0);
+            bf16x8 a2 = lds_operand_tr(Qs, QS, r0 + kb * 16, db * 32, lane);
+            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, dsb, dkacc[db], 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int r = kb * 8 + e;
+            const int qi = r0 + 8 * (r / 4) + 4 * hh + (r % 4);
+            dSs[qi * DSS + wkey + l32] = dsb[e];
+        }
+    }
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
-    constexpr int BN = 128;      // keys per block, 32 per wave
-    constexpr int BM = 32;       // query rows per iteration
-    constexpr int QS = D + 8;    // Q / dO tile row stride (elements)
-    constexpr int DSS = BN + 8;  // dS tile row stride
+    using L = BwdLds<D>;
+    constexpr int BN = L::BN, BM = L::BM, QS = L::QS, DSS = L::DSS;
     constexpr int CPR = D / 8;
-    constexpr int NLD = BM * CPR / 256;  // 16-byte chunks per thread per tile (2 for D=128, 1 for D=64)
-    static_assert(NLD >= 1, "tile too small");
-    __shared__ __attribute__((aligned(16))) __bf16 Qs[BM * QS];
-    __shared__ __attribute__((aligned(16))) __bf16 dOs[BM * QS];
-    __shared__ __attribute__((aligned(16))) __bf16 dSs[BM * DSS];
-    __shared__ __attribute__((aligned(16))) float lse_s[BM];
-    __shared__ __attribute__((aligned(16))) float dlt_s[BM];
+    constexpr int NLD = BM * CPR / 256;  // 16-byte chunks per thread per tile (4 for D=128, 2 for D=64)
+    constexpr int RPL = 256 / CPR;       // rows covered by one pass of the block's 256 threads
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hh = lane >> 5;
     const bool causal = p.flags & LTR_CAUSAL;
 
@@ -578,11 +651,13 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
     if (c >= p.n_chunks) return;
     const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
     const int key0 = kt * BN;
-    const int my_key = key0 + w * 32 + l32;     // this lane's key in S / dP / dK^T / dV^T tiles
+    const int wkey = w * 32;
+    const int my_key = key0 + wkey + l32;       // this lane's key in S / dP / dK^T / dV^T tiles
     const bool key_ok = my_key < sk;
     const int my_kpos = pos0 + my_key;
     const int tile_kpos_lo = pos0 + key0;
     const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
+    const bool key_tail = key0 + BN > sk;
 
     // resident operands.  kreg / vreg: B operand of S = Q K^T and dP = dO V^T, lane (key l32,
     // half hh) holds d = 16*kb + 8*hh .. +7.  ktreg: B operand of dQ = dS K over this wave's
@@ -591,145 +666,168 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
     {
         const __bf16 *kp = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
         const __bf16 *vp = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+        const int ksafe = min(my_key, sk - 1);
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
-            uint4 kx = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0);
-            if (key_ok) {
-                kx = *(const uint4 *)(kp + (long long)my_key * p.ks[1] + kb * 16 + 8 * hh);
-                vx = *(const uint4 *)(vp + (long long)my_key * p.vs[1] + kb * 16 + 8 * hh);
+            uint4 kx = *(const uint4 *)(kp + (long long)ksafe * p.ks[1] + kb * 16 + 8 * hh);
+            uint4 vx = *(const uint4 *)(vp + (long long)ksafe * p.vs[1] + kb * 16 + 8 * hh);
+            if (!key_ok) {
+                kx = make_uint4(0, 0, 0, 0);
+                vx = make_uint4(0, 0, 0, 0);
             }
             kreg[kb] = as_bf16x8(kx);
             vreg[kb] = as_bf16x8(vx);
         }
-        const int dcol = (w * 32 + l32) % D;  // D = 64: waves 2,3 repeat columns 0..63 (results unused)
+        const int dcol = (wkey + l32) % D;  // D = 64: waves 2,3 repeat columns 0..63 (results unused)
 #pragma unroll
         for (int kb = 0; kb < BN / 16; kb++) {
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                int key = key0 + kb * 16 + 8 * hh + e;
-                ktreg[kb][e] = key < sk ? kp[(long long)key * p.ks[1] + dcol] : (__bf16)0.f;
+                const int key = key0 + kb * 16 + 8 * hh + e;
+                const __bf16 x = kp[(long long)min(key, sk - 1) * p.ks[1] + dcol];
+                ktreg[kb][e] = key < sk ? x : (__bf16)0.f;
             }
         }
     }
 
+    f32x16 zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
     f32x16 dkacc[D / 32], dvacc[D / 32];
 #pragma unroll
-    for (int i = 0; i < D / 32; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            dkacc[i][r] = 0.f;
-            dvacc[i][r] = 0.f;
-        }
+    for (int i = 0; i < D / 32; i++) {
+        dkacc[i] = zero16;
+        dvacc[i] = zero16;
+    }
     const float c2 = p.scale * LTR_LOG2E;
 
-    for (int rep = 0; rep < p.n_rep; rep++) {
-        const int h = hkv * p.n_rep + rep;
-        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
-        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
-        const float *lsep = p.lse + ((long long)b * p.Hq + h) * p.Sq;
-        const float *dltp = p.delta + ((long long)b * p.Hq + h) * p.Sq;
-        float *dqp = p.dq + b * p.dqs[0] + h * p.dqs[2];
-        for (int qt = 0; qt < p.n_qtiles; qt++) {
-            const int row0 = qt * BM;
-            int t_lo, t_hi;
-            q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], t_lo, t_hi);
-            if (causal && t_hi < tile_kpos_lo) continue;  // no query of the tile sees any key of the block
-            __syncthreads();
+    // iteration space: (query head of the group, 64-row query tile), invisible tiles skipped
+    const int n_it = p.n_rep * p.n_qtiles;
+    auto tile_visible = [&](int it) {
+        if (!causal) return true;
+        const int row0 = (it % p.n_qtiles) * BM;
+        int lo, hi;
+        q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
+        return hi >= tile_kpos_lo;
+    };
+    auto next_visible = [&](int it) {
+        while (it < n_it && !tile_visible(it)) it++;
+        return it;
+    };
+
+    // per-thread staging coordinates: row (tid / CPR) + RPL*i, 16-byte chunk tid % CPR
+    const int ld_r = tid / CPR, ld_c = tid % CPR;
+    const unsigned q_voff = (unsigned)(ld_r * (int)p.qs[1] + ld_c * 8);
+    const unsigned do_voff = (unsigned)(ld_r * (int)p.dos[1] + ld_c * 8);
+    uint4 qld[NLD], dld[NLD];
+    float sld = 0.f;  // threads 0..63: LSE*log2e of row tid; threads 64..127: DELTA of row tid-64
+    auto gload = [&](int it) {
+        const int h = hkv * p.n_rep + it / p.n_qtiles;
+        const int row0 = (it % p.n_qtiles) * BM;
+        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2] + (long long)row0 * p.qs[1];
+        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2] + (long long)row0 * p.dos[1];
+        const float *lsep = p.lse + ((long long)b * p.Hq + h) * p.Sq + row0;
+        const float *dltp = p.delta + ((long long)b * p.Hq + h) * p.Sq + row0;
+        if (row0 + BM <= p.Sq) {
 #pragma unroll
             for (int i = 0; i < NLD; i++) {
-                int id = tid + 256 * i;
-                int r = id / CPR, dc = id % CPR;
-                uint4 qx = make_uint4(0, 0, 0, 0), dx = make_uint4(0, 0, 0, 0);
-                if (row0 + r < p.Sq) {
-                    qx = *(const uint4 *)(qp + (long long)(row0 + r) * p.qs[1] + dc * 8);
-                    dx = *(const uint4 *)(dop + (long long)(row0 + r) * p.dos[1] + dc * 8);
+                qld[i] = *(const uint4 *)(qp + (q_voff + (unsigned)(i * RPL * (int)p.qs[1])));
+                dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
+            }
+            if (tid < BM) sld = lsep[tid] * LTR_LOG2E;
+            else if (tid < 2 * BM) sld = dltp[tid - BM];
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                qld[i] = make_uint4(0, 0, 0, 0);
+                dld[i] = make_uint4(0, 0, 0, 0);
+                if (row0 + ld_r + i * RPL < p.Sq) {
+                    qld[i] = *(const uint4 *)(qp + (q_voff + (unsigned)(i * RPL * (int)p.qs[1])));
+                    dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
                 }
-                *(uint4 *)(Qs + r * QS + dc * 8) = qx;
-                *(uint4 *)(dOs + r * QS + dc * 8) = dx;
             }
-            if (tid < BM) {
-                lse_s[tid] = (row0 + tid < p.Sq) ? lsep[row0 + tid] : INFINITY;
-            } else if (tid < 2 * BM) {
-                dlt_s[tid - BM] = (row0 + tid - BM < p.Sq) ? dltp[row0 + tid - BM] : 0.f;
-            }
-            __syncthreads();
+            // rows past the end: LSE = +inf makes P = 0
+            if (tid < BM) sld = (row0 + tid < p.Sq) ? lsep[tid] * LTR_LOG2E : INFINITY;
+            else if (tid < 2 * BM) sld = (row0 + tid - BM < p.Sq) ? dltp[tid - BM] : 0.f;
+        }
+    };
+    auto lds_store = [&](int buf) {
+        __bf16 *Qs = (__bf16 *)(smem + buf * L::BUF_BYTES);
+        __bf16 *dOs = Qs + L::TILE;
+        float *st = (float *)(dOs + L::TILE);
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            *(uint4 *)(Qs + (ld_r + i * RPL) * QS + ld_c * 8) = qld[i];
+            *(uint4 *)(dOs + (ld_r + i * RPL) * QS + ld_c * 8) = dld[i];
+        }
+        if (tid < 2 * BM) st[tid] = sld;
+    };
 
-            // wave-uniform skip: none of this wave's keys is visible to any row of the tile
-            const bool wave_active = !causal || (pos0 + key0 + w * 32 <= t_hi);
-            f32x16 s, dp;
+    int it = next_visible(0);
+    if (it < n_it) {
+        gload(it);
+        lds_store(0);
+    }
+    __syncthreads();
+    int par = 0;
+    const int dq_lane = 4 * hh * (int)p.dqs[1] + wkey + l32;   // this lane's element offset inside a dQ sub-tile
+    while (it < n_it) {
+        const int it_next = next_visible(it + 1);
+        if (it_next < n_it) gload(it_next);
+
+        const int h = hkv * p.n_rep + it / p.n_qtiles;
+        const int row0 = (it % p.n_qtiles) * BM;
+        const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
+        const __bf16 *dOs = Qs + L::TILE;
+        const float *lse_s = (const float *)(dOs + L::TILE);
+        const float *dlt_s = lse_s + BM;
+        __bf16 *dSs = (__bf16 *)(smem + 2 * L::BUF_BYTES + par * L::DS_BYTES);
+
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                s[r] = 0.f;
-                dp[r] = 0.f;
-            }
-            if (wave_active) {
+        for (int sub = 0; sub < 2; sub++) {
+            const int r0 = sub * 32;
+            int t_lo, t_hi;
+            const int srow1 = min(row0 + r0 + 32, p.Sq) - 1;
+            if (srow1 >= row0 + r0) q_pos_range(row0 + r0, srow1, p.q_split, p.q_pos0[0], p.q_pos0[1], t_lo, t_hi);
+            else { t_lo = -0x7fffffff; t_hi = -0x7fffffff; }   // no rows: everything masked
+            const bool need_mask = key_tail || (row0 + r0 + 32 > p.Sq) || (causal && tile_kpos_hi > t_lo);
+            bwd_sub_tile<D>(Qs, dOs, lse_s, dlt_s, dSs, kreg, vreg, dkacc, dvacc, zero16, r0, lane, l32, hh, wkey, c2,
+                            need_mask, key_ok, causal, my_kpos, row0, p.Sq, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+        }
+        if (it_next < n_it) lds_store(par ^ 1);
+        __syncthreads();
+        // dQ[:, 32w .. 32w+31] = dS (64 x 128 keys) K[:, 32w ..]
+        if (wkey < D) {
+            float *dqp = p.dq + b * p.dqs[0] + h * p.dqs[2] + (long long)row0 * p.dqs[1];
 #pragma unroll
-                for (int kb = 0; kb < D / 16; kb++) {
-                    bf16x8 a = *(const bf16x8 *)(Qs + l32 * QS + kb * 16 + 8 * hh);
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kreg[kb], s, 0, 0, 0);
-                }
-#pragma unroll
-                for (int kb = 0; kb < D / 16; kb++) {
-                    bf16x8 a = *(const bf16x8 *)(dOs + l32 * QS + kb * 16 + 8 * hh);
-                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vreg[kb], dp, 0, 0, 0);
-                }
-                const bool need_mask = (key0 + BN > sk) || (causal && tile_kpos_hi > t_lo);
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f32x4 lv = *(const f32x4 *)(lse_s + 8 * g + 4 * hh);
-                    const f32x4 dv = *(const f32x4 *)(dlt_s + 8 * g + 4 * hh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int r = 4 * g + e;
-                        float pv = exp2f(s[r] * c2 - lv[e] * LTR_LOG2E);
-                        if (need_mask) {
-                            const int qrow = row0 + 8 * g + 4 * hh + e;
-                            const int qpos = q_position(qrow, p.q_split, p.q_pos0[0], p.q_pos0[1]);
-                            const bool vis = key_ok && (!causal || my_kpos <= qpos);
-                            pv = vis ? pv : 0.f;
-                        }
-                        s[r] = pv;
-                        dp[r] = pv * (dp[r] - dv[e]);
-                    }
-                }
-                // dV^T += dO^T P and dK^T += Q^T dS: contraction over the 32 query rows
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++) {
-                    bf16x8 pb = pack_bf16x8(s, kb * 8);
-                    bf16x8 dsb = pack_bf16x8(dp, kb * 8);
-#pragma unroll
-                    for (int db = 0; db < D / 32; db++) {
-                        bf16x8 a = lds_operand_tr(dOs, QS, kb * 16, db * 32, lane);
-                        dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, dvacc[db], 0, 0, 0);
-                        bf16x8 a2 = lds_operand_tr(Qs, QS, kb * 16, db * 32, lane);
-                        dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, dsb, dkacc[db], 0, 0, 0);
-                    }
-                }
-            }
-            // dS tile [query][key] to LDS (zeros from inactive waves)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int qi = 8 * (r / 4) + 4 * hh + (r % 4);
-                dSs[qi * DSS + w * 32 + l32] = (__bf16)dp[r];
-            }
-            __syncthreads();
-            // dQ[:, 32w .. 32w+31] = dS (32 x 128 keys) K[:, 32w ..]
-            if (w * 32 < D) {
-                f32x16 dq;
-#pragma unroll
-                for (int r = 0; r < 16; r++) dq[r] = 0.f;
+            for (int sub = 0; sub < 2; sub++) {
+                const int r0 = sub * 32;
+                if (row0 + r0 >= p.Sq) break;
+                f32x16 dq = zero16;
 #pragma unroll
                 for (int kb = 0; kb < BN / 16; kb++) {
-                    bf16x8 a = *(const bf16x8 *)(dSs + l32 * DSS + kb * 16 + 8 * hh);
+                    bf16x8 a = *(const bf16x8 *)(dSs + (r0 + l32) * DSS + kb * 16 + 8 * hh);
                     dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, ktreg[kb], dq, 0, 0, 0);
                 }
+                float *dqs = dqp + (long long)r0 * p.dqs[1];
+                if (row0 + r0 + 32 <= p.Sq) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int qrow = row0 + 8 * (r / 4) + 4 * hh + (r % 4);
-                    if (qrow < p.Sq) atomicAdd(dqp + (long long)qrow * p.dqs[1] + w * 32 + l32, dq[r] * p.scale);
+                    for (int r = 0; r < 16; r++) {
+                        const int roff = (8 * (r / 4) + (r % 4)) * (int)p.dqs[1];   // uniform
+                        atomicAdd(dqs + (unsigned)(dq_lane + roff), dq[r] * p.scale);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int qrow = row0 + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
+                        const int roff = (8 * (r / 4) + (r % 4)) * (int)p.dqs[1];
+                        if (qrow < p.Sq) atomicAdd(dqs + (unsigned)(dq_lane + roff), dq[r] * p.scale);
+                    }
                 }
             }
         }
+        it = it_next;
+        par ^= 1;
     }
 
     // dK^T / dV^T tiles: lane (key l32 of this wave, half hh), register r -> d = 32*db + 8*(r/4) + 4hh + r%4
@@ -767,6 +865,19 @@ int check_device() {
         cached = (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') ? 1 : -1;
     }
     return cached == 1 ? LTR_OK : LTR_EDEVICE;
+}
+
+// kernels that need more than 64 KB of dynamic LDS must opt in once per process
+int enable_large_lds() {
+    static int done = 0;  // 0 not yet, 1 ok, -1 failed
+    if (done == 0) {
+        bool ok = hipFuncSetAttribute((const void *)bwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      BwdLds<128>::TOTAL) == hipSuccess &&
+                  hipFuncSetAttribute((const void *)bwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      BwdLds<64>::TOTAL) == hipSuccess;
+        done = ok ? 1 : -1;
+    }
+    return done == 1 ? LTR_OK : LTR_ELAUNCH;
 }
 
 bool strides_ok(const int64_t *s, int elem_bytes) {
@@ -936,7 +1047,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     p.Hkv = a->Hkv;
     p.n_rep = a->Hq / a->Hkv;
     p.Sq = (int)a->Sq;
-    p.n_qtiles = (p.Sq + 31) / 32;
+    p.n_qtiles = (p.Sq + 63) / 64;
     for (int i = 0; i < 3; i++) {
         p.qs[i] = a->q_stride[i];
         p.dos[i] = a->do_stride[i];
@@ -956,8 +1067,10 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     const long long nblk = tiles * p.B * p.Hkv;
     if (nblk > 0x7fffffffLL) return LTR_EINVAL;
     hipStream_t st = (hipStream_t)stream;
-    if (a->D == 128) hipLaunchKernelGGL(bwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL(bwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), 0, st, p);
+    rc = enable_large_lds();
+    if (rc) return rc;
+    if (a->D == 128) hipLaunchKernelGGL(bwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), BwdLds<128>::TOTAL, st, p);
+    else hipLaunchKernelGGL(bwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), BwdLds<64>::TOTAL, st, p);
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
 
