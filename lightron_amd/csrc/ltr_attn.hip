@@ -11,17 +11,19 @@
 //                        result is part of the epilogue.
 //   fwd_f32_kernel<D>    fp32 I/O and arithmetic (no MFMA), for the 1e-4 parity case.
 //   delta_kernel         DELTA = rowsum(dO * O).
-//   bwd_bf16_kernel<D>   a block owns 128 keys of one kv head (32 per wave, K and V operands
+//   bwd_dkdv_kernel<D>   a block owns 128 keys of one kv head (32 per wave, K and V operands
 //                        resident in registers), loops over the query heads of the GQA group
-//                        and over query tiles; dK^T/dV^T accumulate in registers, dS goes
-//                        through LDS so each wave forms a complete 32x32 slice of dQ, which is
-//                        added to the fp32 accumulator in HBM with hardware float atomics.
+//                        and over query tiles; dK^T/dV^T accumulate in registers.
+//   bwd_dq_kernel<D>     forward-shaped: a block owns 128 query rows, loops over K/V tiles,
+//                        dQ^T accumulates in registers.  No atomics anywhere: results are
+//                        bitwise reproducible.
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, i = l % 32, h = l / 32):
 //   A[i][8h .. 8h+7], B[8h .. 8h+7][i], C[8*(r/4) + 4h + r%4][i] for accumulator register r.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <math.h>
+#include <type_traits>
 #include "ltr_attn.h"
 
 namespace {
@@ -538,31 +540,37 @@ __global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst
 }
 
 // ------------------------------------------------------------------------------ backward, bf16
-// LDS (dynamic): two buffers of {Q tile, dO tile, LSE*log2e, DELTA} for 64 query rows, two dS tiles.
+// Two kernels, no atomics, bitwise reproducible:
+//   bwd_dkdv_kernel  a block owns 128 keys of one kv head (32 per wave; K and V operands live in
+//                    registers), loops over the query heads of the GQA group and over 64-row
+//                    query tiles staged in double-buffered LDS; dK^T and dV^T accumulate in
+//                    registers for the whole loop and are added to the fp32 accumulators once.
+//   bwd_dq_kernel    a block owns 128 query rows of one query head (32 per wave; Q and dO
+//                    operands in registers), loops over 64-key K/V tiles like the forward;
+//                    dQ^T accumulates in registers.
+// LDS of bwd_dkdv_kernel (dynamic): two buffers of {Q tile, dO tile, LSE*log2e, DELTA}.
 template <int D>
 struct BwdLds {
     static constexpr int BN = 128;      // keys per block, 32 per wave
     static constexpr int BM = 64;       // query rows per iteration (two 32-row MFMA sub-tiles)
     static constexpr int QS = D + 8;    // Q / dO tile row stride (elements)
-    static constexpr int DSS = BN + 8;  // dS tile row stride
     static constexpr int TILE = BM * QS;                                 // elements
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, lse, delta
-    static constexpr int DS_BYTES = BM * DSS * 2;
-    static constexpr int TOTAL = 2 * BUF_BYTES + 2 * DS_BYTES;
+    static constexpr int TOTAL = 2 * BUF_BYTES;
 };
 
-// One 32-row sub-tile of the backward for one wave (its 32 keys): S and dP by MFMA, P and dS in
-// registers, dV^T / dK^T accumulation, dS written to LDS as [query][key].  Straight-line code
-// around the accumulators: the mask (diagonal and edge tiles only) is a fix-up of P and dS under
-// a wave-uniform branch, so dkacc / dvacc never cross a control-flow merge.
-template <int D>
-__device__ __forceinline__ void bwd_sub_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
-                                             __bf16 *dSs, const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16],
-                                             f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &zero16,
-                                             int r0, int lane, int l32, int hh, int wkey, float c2, bool need_mask,
-                                             bool key_ok, bool causal, int my_kpos, int row_base, int Sq, int q_split,
-                                             int p0, int p1) {
-    constexpr int QS = BwdLds<D>::QS, DSS = BwdLds<D>::DSS;
+// One 32-row sub-tile for one wave (its 32 keys): S = Q K^T and dP = dO V^T by MFMA (query rows in
+// accumulator registers, this lane's key in the lane), P = exp2(S*c2 - LSE*log2e), dS = P*(dP - DELTA),
+// then dV^T += dO^T P and dK^T += Q^T dS with P / dS fed from registers as B operands and dO^T / Q^T
+// read from the same LDS tiles by transpose loads.
+template <int D, bool MASK>
+__device__ __forceinline__ void bwd_dkdv_sub_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s,
+                                                  const float *dlt_s, const bf16x8 (&kreg)[D / 16],
+                                                  const bf16x8 (&vreg)[D / 16], f32x16 (&dkacc)[D / 32],
+                                                  f32x16 (&dvacc)[D / 32], const f32x16 &zero16, int r0, int lane, int l32,
+                                                  int hh, float c2, bool key_ok, bool causal, int my_kpos, int row_base,
+                                                  int Sq, int q_split, int p0, int p1) {
+    constexpr int QS = BwdLds<D>::QS;
     f32x16 s = zero16, dp = zero16;
 #pragma unroll
     for (int kb = 0; kb < D / 16; kb++) {
@@ -581,19 +589,17 @@ __device__ __forceinline__ void bwd_sub_tile(const __bf16 *Qs, const __bf16 *dOs
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const int r = 4 * g + e;
-            const float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lv[e]);
+            float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lv[e]);
+            float dsv = pv * (dp[r] - dv[e]);
+            if (MASK) {
+                const int qrow = row_base + r0 + 8 * g + 4 * hh + e;
+                const int qpos = q_position(qrow, q_split, p0, p1);
+                const bool vis = key_ok && qrow < Sq && (!causal || my_kpos <= qpos);
+                pv = vis ? pv : 0.f;
+                dsv = vis ? dsv : 0.f;
+            }
             s[r] = pv;
-            dp[r] = pv * (dp[r] - dv[e]);
-        }
-    }
-    if (need_mask) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int qrow = row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
-            const int qpos = q_position(qrow, q_split, p0, p1);
-            const bool vis = key_ok && qrow < Sq && (!causal || my_kpos <= qpos);
-            s[r] = vis ? s[r] : 0.f;
-            dp[r] = vis ? dp[r] : 0.f;
+            dp[r] = dsv;
         }
     }
 #pragma unroll
@@ -607,19 +613,13 @@ __device__ __forceinline__ void bwd_sub_tile(const __bf16 *Qs, const __bf16 *dOs
             bf16x8 a2 = lds_operand_tr(Qs, QS, r0 + kb * 16, db * 32, lane);
             dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, dsb, dkacc[db], 0, 0, 0);
         }
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const int r = kb * 8 + e;
-            const int qi = r0 + 8 * (r / 4) + 4 * hh + (r % 4);
-            dSs[qi * DSS + wkey + l32] = dsb[e];
-        }
     }
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
+__global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     using L = BwdLds<D>;
-    constexpr int BN = L::BN, BM = L::BM, QS = L::QS, DSS = L::DSS;
+    constexpr int BN = L::BN, BM = L::BM, QS = L::QS;
     constexpr int CPR = D / 8;
     constexpr int NLD = BM * CPR / 256;  // 16-byte chunks per thread per tile (4 for D=128, 2 for D=64)
     constexpr int RPL = 256 / CPR;       // rows covered by one pass of the block's 256 threads
@@ -651,18 +651,15 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
     if (c >= p.n_chunks) return;
     const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
     const int key0 = kt * BN;
-    const int wkey = w * 32;
-    const int my_key = key0 + wkey + l32;       // this lane's key in S / dP / dK^T / dV^T tiles
+    const int my_key = key0 + w * 32 + l32;     // this lane's key in S / dP / dK^T / dV^T tiles
     const bool key_ok = my_key < sk;
     const int my_kpos = pos0 + my_key;
     const int tile_kpos_lo = pos0 + key0;
     const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
     const bool key_tail = key0 + BN > sk;
 
-    // resident operands.  kreg / vreg: B operand of S = Q K^T and dP = dO V^T, lane (key l32,
-    // half hh) holds d = 16*kb + 8*hh .. +7.  ktreg: B operand of dQ = dS K over this wave's
-    // 32 columns of D (d = 32*w + l32) and all 128 keys: K-dim values are keys 16*kb + 8*hh + e.
-    bf16x8 kreg[D / 16], vreg[D / 16], ktreg[BN / 16];
+    // resident B operands of S = Q K^T and dP = dO V^T: lane (key l32, half hh) holds d = 16*kb + 8*hh .. +7
+    bf16x8 kreg[D / 16], vreg[D / 16];
     {
         const __bf16 *kp = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
         const __bf16 *vp = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
@@ -678,16 +675,6 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
             kreg[kb] = as_bf16x8(kx);
             vreg[kb] = as_bf16x8(vx);
         }
-        const int dcol = (wkey + l32) % D;  // D = 64: waves 2,3 repeat columns 0..63 (results unused)
-#pragma unroll
-        for (int kb = 0; kb < BN / 16; kb++) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int key = key0 + kb * 16 + 8 * hh + e;
-                const __bf16 x = kp[(long long)min(key, sk - 1) * p.ks[1] + dcol];
-                ktreg[kb][e] = key < sk ? x : (__bf16)0.f;
-            }
-        }
     }
 
     f32x16 zero16;
@@ -701,17 +688,20 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
     }
     const float c2 = p.scale * LTR_LOG2E;
 
-    // iteration space: (query head of the group, 64-row query tile), invisible tiles skipped
+    // iteration space: (query head of the group, 64-row query tile).  Class 0: no row sees any key of
+    // the block (skipped); 1: every (row, key) pair is visible; 2: needs the mask (diagonal, tails).
     const int n_it = p.n_rep * p.n_qtiles;
-    auto tile_visible = [&](int it) {
-        if (!causal) return true;
+    auto tile_class = [&](int it) {
         const int row0 = (it % p.n_qtiles) * BM;
+        const bool edge = key_tail || row0 + BM > p.Sq;
+        if (!causal) return edge ? 2 : 1;
         int lo, hi;
         q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
-        return hi >= tile_kpos_lo;
+        if (hi < tile_kpos_lo) return 0;
+        return (edge || tile_kpos_hi > lo) ? 2 : 1;
     };
-    auto next_visible = [&](int it) {
-        while (it < n_it && !tile_visible(it)) it++;
+    auto next_of = [&](int it, int cls) {
+        while (it < n_it && tile_class(it) != cls) it++;
         return it;
     };
 
@@ -746,7 +736,7 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
                     dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
                 }
             }
-            // rows past the end: LSE = +inf makes P = 0
+            // rows past the end: LSE = +inf makes P = 0 (they are masked as well)
             if (tid < BM) sld = (row0 + tid < p.Sq) ? lsep[tid] * LTR_LOG2E : INFINITY;
             else if (tid < 2 * BM) sld = (row0 + tid - BM < p.Sq) ? dltp[tid - BM] : 0.f;
         }
@@ -763,72 +753,39 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
         if (tid < 2 * BM) st[tid] = sld;
     };
 
-    int it = next_visible(0);
-    if (it < n_it) {
+    // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
+    // live in straight-line loop bodies
+    auto run_pass = [&](auto mask_tag) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr int cls = MASK ? 2 : 1;
+        int it = next_of(0, cls);
+        if (it >= n_it) return;
+        __syncthreads();   // the previous pass has finished reading LDS
         gload(it);
         lds_store(0);
-    }
-    __syncthreads();
-    int par = 0;
-    const int dq_lane = 4 * hh * (int)p.dqs[1] + wkey + l32;   // this lane's element offset inside a dQ sub-tile
-    while (it < n_it) {
-        const int it_next = next_visible(it + 1);
-        if (it_next < n_it) gload(it_next);
-
-        const int h = hkv * p.n_rep + it / p.n_qtiles;
-        const int row0 = (it % p.n_qtiles) * BM;
-        const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
-        const __bf16 *dOs = Qs + L::TILE;
-        const float *lse_s = (const float *)(dOs + L::TILE);
-        const float *dlt_s = lse_s + BM;
-        __bf16 *dSs = (__bf16 *)(smem + 2 * L::BUF_BYTES + par * L::DS_BYTES);
-
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
-            const int r0 = sub * 32;
-            int t_lo, t_hi;
-            const int srow1 = min(row0 + r0 + 32, p.Sq) - 1;
-            if (srow1 >= row0 + r0) q_pos_range(row0 + r0, srow1, p.q_split, p.q_pos0[0], p.q_pos0[1], t_lo, t_hi);
-            else { t_lo = -0x7fffffff; t_hi = -0x7fffffff; }   // no rows: everything masked
-            const bool need_mask = key_tail || (row0 + r0 + 32 > p.Sq) || (causal && tile_kpos_hi > t_lo);
-            bwd_sub_tile<D>(Qs, dOs, lse_s, dlt_s, dSs, kreg, vreg, dkacc, dvacc, zero16, r0, lane, l32, hh, wkey, c2,
-                            need_mask, key_ok, causal, my_kpos, row0, p.Sq, p.q_split, p.q_pos0[0], p.q_pos0[1]);
-        }
-        if (it_next < n_it) lds_store(par ^ 1);
         __syncthreads();
-        // dQ[:, 32w .. 32w+31] = dS (64 x 128 keys) K[:, 32w ..]
-        if (wkey < D) {
-            float *dqp = p.dq + b * p.dqs[0] + h * p.dqs[2] + (long long)row0 * p.dqs[1];
+        int par = 0;
+        while (it < n_it) {
+            const int it_next = next_of(it + 1, cls);
+            if (it_next < n_it) gload(it_next);
+            const int row0 = (it % p.n_qtiles) * BM;
+            const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
+            const __bf16 *dOs = Qs + L::TILE;
+            const float *lse_s = (const float *)(dOs + L::TILE);
+            const float *dlt_s = lse_s + BM;
 #pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
-                const int r0 = sub * 32;
-                if (row0 + r0 >= p.Sq) break;
-                f32x16 dq = zero16;
-#pragma unroll
-                for (int kb = 0; kb < BN / 16; kb++) {
-                    bf16x8 a = *(const bf16x8 *)(dSs + (r0 + l32) * DSS + kb * 16 + 8 * hh);
-                    dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, ktreg[kb], dq, 0, 0, 0);
-                }
-                float *dqs = dqp + (long long)r0 * p.dqs[1];
-                if (row0 + r0 + 32 <= p.Sq) {
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int roff = (8 * (r / 4) + (r % 4)) * (int)p.dqs[1];   // uniform
-                        atomicAdd(dqs + (unsigned)(dq_lane + roff), dq[r] * p.scale);
-                    }
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int qrow = row0 + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
-                        const int roff = (8 * (r / 4) + (r % 4)) * (int)p.dqs[1];
-                        if (qrow < p.Sq) atomicAdd(dqs + (unsigned)(dq_lane + roff), dq[r] * p.scale);
-                    }
-                }
-            }
+            for (int sub = 0; sub < 2; sub++)
+                bwd_dkdv_sub_tile<D, MASK>(Qs, dOs, lse_s, dlt_s, kreg, vreg, dkacc, dvacc, zero16, sub * 32, lane, l32,
+                                           hh, c2, key_ok, causal, my_kpos, row0, p.Sq, p.q_split, p.q_pos0[0],
+                                           p.q_pos0[1]);
+            if (it_next < n_it) lds_store(par ^ 1);
+            __syncthreads();
+            it = it_next;
+            par ^= 1;
         }
-        it = it_next;
-        par ^= 1;
-    }
+    };
+    run_pass(std::false_type{});
+    run_pass(std::true_type{});
 
     // dK^T / dV^T tiles: lane (key l32 of this wave, half hh), register r -> d = 32*db + 8*(r/4) + 4hh + r%4
     if (key_ok) {
@@ -847,6 +804,197 @@ __global__ __launch_bounds__(256) void bwd_bf16_kernel(const BwdParams p) {
                 }
                 *(f32x4 *)(dkp + d) = ok;
                 *(f32x4 *)(dvp + d) = ov;
+            }
+    }
+}
+
+// dQ: same block / wave / lane roles as the forward (a lane owns one query row), so LSE and DELTA are
+// per-lane scalars.  S^T = K Q^T and dP^T = V dO^T with K, V tiles natural in LDS; dS^T leaves the
+// registers as the B operand of dQ^T += K^T dS^T, whose A operand is the K tile read by transpose loads.
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdParams p) {
+    constexpr int BM = 128, BN = 64;
+    constexpr int KS = D + 8;
+    constexpr int VS = D + 8;
+    constexpr int CPR = D / 8;
+    constexpr int NLD = BN * CPR / 256;
+    __shared__ __attribute__((aligned(16))) __bf16 Ks[BN * KS];
+    __shared__ __attribute__((aligned(16))) __bf16 Vs[BN * VS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hh = lane >> 5;
+    const bool causal = p.flags & LTR_CAUSAL;
+
+    int idx = blockIdx.x, pair, rest;
+    const int P = p.B * p.Hkv;
+    if ((P & 7) == 0) {
+        int xcd = idx & 7, j = idx >> 3, pp = P >> 3;
+        pair = (j % pp) * 8 + xcd;
+        rest = j / pp;
+    } else {
+        pair = idx % P;
+        rest = idx / P;
+    }
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    const int rep = rest % p.n_rep;
+    const int qt = n_qt - 1 - rest / p.n_rep;
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
+
+    const int row0 = qt * BM;
+    const int my_row = row0 + w * 32 + l32;
+    const bool row_ok = my_row < p.Sq;
+    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int blk_lo, blk_hi, w_lo, w_hi;
+    q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+    {
+        int wr0 = row0 + w * 32, wr1 = min(wr0 + 32, p.Sq) - 1;
+        if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
+        else { w_lo = -0x7fffffff; w_hi = -0x7fffffff; }  // wave has no valid row: everything masked
+    }
+
+    bf16x8 qreg[D / 16], doreg[D / 16];
+    float lse2 = INFINITY, dlt = 0.f;
+    {
+        const int rsafe = min(my_row, p.Sq - 1);
+        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + (long long)rsafe * p.qs[1] + h * p.qs[2];
+        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + (long long)rsafe * p.dos[1] + h * p.dos[2];
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) {
+            qreg[kb] = as_bf16x8(*(const uint4 *)(qp + kb * 16 + 8 * hh));
+            doreg[kb] = as_bf16x8(*(const uint4 *)(dop + kb * 16 + 8 * hh));
+        }
+        if (row_ok) {
+            lse2 = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row] * LTR_LOG2E;
+            dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
+        }
+    }
+    f32x16 zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+    f32x16 dqacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; i++) dqacc[i] = zero16;
+    const float c2 = p.scale * LTR_LOG2E;
+
+    int c = 0, t = 0, nt = 0;
+    auto ntiles_of = [&](int ci) {
+        int sk = p.chunk[ci].sk;
+        int nvis = causal ? max(0, min(sk, blk_hi - p.chunk[ci].pos0 + 1)) : sk;
+        return (nvis + BN - 1) / BN;
+    };
+    auto settle = [&]() {
+        while (c < p.n_chunks && t >= nt) {
+            c++;
+            t = 0;
+            if (c < p.n_chunks) nt = ntiles_of(c);
+        }
+    };
+    nt = ntiles_of(0);
+    settle();
+
+    const int ld_r = tid / CPR, ld_c = tid % CPR;
+    constexpr int RPL = 256 / CPR;
+    uint4 kld[NLD], vld[NLD];
+    auto gload = [&](int ci, int ti) {
+        const int sk = p.chunk[ci].sk;
+        const __bf16 *kp = (const __bf16 *)p.chunk[ci].k + b * p.ks[0] + hkv * p.ks[2] + (long long)(ti * BN) * p.ks[1];
+        const __bf16 *vp = (const __bf16 *)p.chunk[ci].v + b * p.vs[0] + hkv * p.vs[2] + (long long)(ti * BN) * p.vs[1];
+        const unsigned kvo = (unsigned)(ld_r * (int)p.ks[1] + ld_c * 8), vvo = (unsigned)(ld_r * (int)p.vs[1] + ld_c * 8);
+        if (ti * BN + BN <= sk) {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                kld[i] = *(const uint4 *)(kp + (kvo + (unsigned)(i * RPL * (int)p.ks[1])));
+                vld[i] = *(const uint4 *)(vp + (vvo + (unsigned)(i * RPL * (int)p.vs[1])));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                kld[i] = make_uint4(0, 0, 0, 0);
+                vld[i] = make_uint4(0, 0, 0, 0);
+                if (ti * BN + ld_r + i * RPL < sk) {
+                    kld[i] = *(const uint4 *)(kp + (kvo + (unsigned)(i * RPL * (int)p.ks[1])));
+                    vld[i] = *(const uint4 *)(vp + (vvo + (unsigned)(i * RPL * (int)p.vs[1])));
+                }
+            }
+        }
+    };
+
+    bool have = c < p.n_chunks;
+    if (have) gload(c, t);
+    while (have) {
+        const int cc = c, ct = t;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            *(uint4 *)(Ks + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
+            *(uint4 *)(Vs + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
+        }
+        __syncthreads();
+        t++;
+        settle();
+        const bool have_next = c < p.n_chunks;
+        if (have_next) gload(c, t);
+
+        const int sk = p.chunk[cc].sk, pos0 = p.chunk[cc].pos0;
+        const int key0 = ct * BN;
+        f32x16 s[2], dp[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            s[nb] = zero16;
+            dp[nb] = zero16;
+#pragma unroll
+            for (int kb = 0; kb < D / 16; kb++) {
+                bf16x8 a = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
+                s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
+            }
+#pragma unroll
+            for (int kb = 0; kb < D / 16; kb++) {
+                bf16x8 a = *(const bf16x8 *)(Vs + (nb * 32 + l32) * VS + kb * 16 + 8 * hh);
+                dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, doreg[kb], dp[nb], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float pv = __builtin_amdgcn_exp2f(s[nb][r] * c2 - lse2);
+                dp[nb][r] = pv * (dp[nb][r] - dlt);
+            }
+        const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
+        if (need_mask) {
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                    const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
+                    dp[nb][r] = vis ? dp[nb][r] : 0.f;
+                }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
+            bf16x8 dsb = pack_bf16x8(dp[kb >> 1], (kb & 1) * 8);
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+                bf16x8 a = lds_operand_tr(Ks, KS, kb * 16, db * 32, lane);
+                dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsb, dqacc[db], 0, 0, 0);
+            }
+        }
+        have = have_next;
+    }
+
+    if (row_ok) {
+        float *dqp = p.dq + b * p.dqs[0] + (long long)my_row * p.dqs[1] + h * p.dqs[2];
+#pragma unroll
+        for (int db = 0; db < D / 32; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = db * 32 + 8 * g + 4 * hh;
+                f32x4 old = *(const f32x4 *)(dqp + d);
+#pragma unroll
+                for (int e = 0; e < 4; e++) old[e] += dqacc[db][4 * g + e] * p.scale;
+                *(f32x4 *)(dqp + d) = old;
             }
     }
 }
@@ -871,9 +1019,9 @@ int check_device() {
 int enable_large_lds() {
     static int done = 0;  // 0 not yet, 1 ok, -1 failed
     if (done == 0) {
-        bool ok = hipFuncSetAttribute((const void *)bwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        bool ok = hipFuncSetAttribute((const void *)bwd_dkdv_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       BwdLds<128>::TOTAL) == hipSuccess &&
-                  hipFuncSetAttribute((const void *)bwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                  hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       BwdLds<64>::TOTAL) == hipSuccess;
         done = ok ? 1 : -1;
     }
@@ -1069,8 +1217,15 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     rc = enable_large_lds();
     if (rc) return rc;
-    if (a->D == 128) hipLaunchKernelGGL(bwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), BwdLds<128>::TOTAL, st, p);
-    else hipLaunchKernelGGL(bwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), BwdLds<64>::TOTAL, st, p);
+    const long long nblk_q = (long long)((p.Sq + 127) / 128) * p.B * p.Hq;
+    if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
+    if (a->D == 128) {
+        hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(256), BwdLds<128>::TOTAL, st, p);
+        hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(256), BwdLds<64>::TOTAL, st, p);
+        hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
+    }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
 
