@@ -164,7 +164,7 @@ template <int D>
 __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     constexpr int BM = 128, BN = 64;
     constexpr int KS = D + 8;    // K tile row stride (elements): natural 128-bit operand reads
-    constexpr int VS = D + 16;   // V tile row stride: transpose reads
+    constexpr int VS = D + 32;   // V tile row stride: transpose reads only (row + 64 B is conflict-free for them)
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int NLD = BN * CPR / 256;
     __shared__ __attribute__((aligned(16))) __bf16 Ks[BN * KS];
@@ -215,14 +215,22 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         }
     }
 
+    f32x16 zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
     f32x16 oacc[D / 32];
 #pragma unroll
-    for (int i = 0; i < D / 32; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
-    float m_run = -INFINITY;  // running max of raw scores (before scale)
+    for (int i = 0; i < D / 32; i++) oacc[i] = zero16;
+    // Online softmax state of this lane's query row.  m_run is the reference point of the exponent
+    // (raw score units); it follows the running max lazily: it moves only when some row of the wave
+    // would otherwise exceed exp2(LTR_LAZY_LOG2) (P stays exactly representable relative to l, which
+    // is accumulated in fp32; LSE = m_run*scale + log(l) is unaffected), so the rescale of the O
+    // accumulator is a rare wave-uniform branch instead of 64 multiplies per tile.
+    float m_run = -INFINITY;
+    float mc = 0.f;           // m_run * c2, or 0 while m_run is still -inf
     float l_run = 0.f;        // this lane's partial row sum (its 32 of the 64 keys per tile)
     const float c2 = p.scale * LTR_LOG2E;
+    constexpr float LAZY = 8.f;
 
     // tile iterator over (chunk, key tile)
     int c = 0, t = 0, nt = 0;
@@ -241,20 +249,30 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     nt = ntiles_of(0);
     settle();
 
+    const int ld_r = tid / CPR, ld_c = tid % CPR;
+    constexpr int RPL = 256 / CPR;
+    const unsigned kvo = (unsigned)(ld_r * (int)p.ks[1] + ld_c * 8), vvo = (unsigned)(ld_r * (int)p.vs[1] + ld_c * 8);
     uint4 kld[NLD], vld[NLD];
     auto gload = [&](int ci, int ti) {
-        const __bf16 *kp = (const __bf16 *)p.chunk[ci].k + b * p.ks[0] + hkv * p.ks[2];
-        const __bf16 *vp = (const __bf16 *)p.chunk[ci].v + b * p.vs[0] + hkv * p.vs[2];
         const int sk = p.chunk[ci].sk;
+        const __bf16 *kp = (const __bf16 *)p.chunk[ci].k + b * p.ks[0] + hkv * p.ks[2] + (long long)(ti * BN) * p.ks[1];
+        const __bf16 *vp = (const __bf16 *)p.chunk[ci].v + b * p.vs[0] + hkv * p.vs[2] + (long long)(ti * BN) * p.vs[1];
+        if (ti * BN + BN <= sk) {
 #pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            int id = tid + 256 * i;
-            int key = ti * BN + id / CPR, dc = id % CPR;
-            kld[i] = make_uint4(0, 0, 0, 0);
-            vld[i] = make_uint4(0, 0, 0, 0);
-            if (key < sk) {
-                kld[i] = *(const uint4 *)(kp + (long long)key * p.ks[1] + dc * 8);
-                vld[i] = *(const uint4 *)(vp + (long long)key * p.vs[1] + dc * 8);
+            for (int i = 0; i < NLD; i++) {
+                kld[i] = *(const uint4 *)(kp + (kvo + (unsigned)(i * RPL * (int)p.ks[1])));
+                vld[i] = *(const uint4 *)(vp + (vvo + (unsigned)(i * RPL * (int)p.vs[1])));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                const bool ok = ti * BN + ld_r + i * RPL < sk;   // the tile's first key always exists
+                kld[i] = *(const uint4 *)(kp + (ok ? kvo + (unsigned)(i * RPL * (int)p.ks[1]) : 0u));
+                vld[i] = *(const uint4 *)(vp + (ok ? vvo + (unsigned)(i * RPL * (int)p.vs[1]) : 0u));
+                if (!ok) {
+                    kld[i] = make_uint4(0, 0, 0, 0);
+                    vld[i] = make_uint4(0, 0, 0, 0);
+                }
             }
         }
     };
@@ -266,10 +284,8 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            int id = tid + 256 * i;
-            int key = id / CPR, dc = id % CPR;
-            *(uint4 *)(Ks + key * KS + dc * 8) = kld[i];
-            *(uint4 *)(Vs + key * VS + dc * 8) = vld[i];
+            *(uint4 *)(Ks + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
+            *(uint4 *)(Vs + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
         }
         __syncthreads();
         t++;
@@ -279,64 +295,63 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
 
         const int sk = p.chunk[cc].sk, pos0 = p.chunk[cc].pos0;
         const int key0 = ct * BN;
-        // wave-uniform: does this wave see any key of the tile at all?
-        const bool wave_active = !causal || (pos0 + key0 <= w_hi);
-        if (wave_active) {
-            f32x16 s[2];
+        f32x16 s[2];
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++) {
+        for (int nb = 0; nb < 2; nb++) {
+            s[nb] = zero16;
 #pragma unroll
-                for (int r = 0; r < 16; r++) s[nb][r] = 0.f;
-#pragma unroll
-                for (int kb = 0; kb < D / 16; kb++) {
-                    bf16x8 a = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
-                    s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
-                }
+            for (int kb = 0; kb < D / 16; kb++) {
+                bf16x8 a = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
+                s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
             }
-            const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
-            if (need_mask) {
-#pragma unroll
-                for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
-                        bool vis = key < sk && (!causal || pos0 + key <= my_pos);
-                        if (!vis) s[nb][r] = -INFINITY;
-                    }
-            }
-            float mx = s[0][0];
-#pragma unroll
-            for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[nb][r]);
-            mx = xhalf_max(mx);
-            const float m_new = fmaxf(m_run, mx);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = exp2f((m_run - m_use) * c2);
-            const float mc = m_use * c2;
-            float psum = 0.f;
+        }
+        // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
+        const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
+        if (need_mask) {
 #pragma unroll
             for (int nb = 0; nb < 2; nb++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    float pv = exp2f(s[nb][r] * c2 - mc);
-                    s[nb][r] = pv;
-                    psum += pv;
+                    const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                    const bool vis = key < sk && (!causal || pos0 + key <= my_pos);
+                    s[nb][r] = vis ? s[nb][r] : -INFINITY;
                 }
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
+        }
+        float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+        for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+        mx = xhalf_max(mx);
+        // move the reference point only when some row needs it
+        const bool grow = (mx > m_run) && (m_run == -INFINITY || (mx - m_run) * c2 > LAZY);
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            const float m_new = fmaxf(m_run, mx);
+            const float mc_new = (m_new == -INFINITY) ? 0.f : m_new * c2;
+            const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mc_new);
+            l_run *= alpha;
 #pragma unroll
             for (int i = 0; i < D / 32; i++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+            m_run = m_new;
+            mc = mc_new;
+        }
+        float psum = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
-                bf16x8 pb = pack_bf16x8(s[kb >> 1], (kb & 1) * 8);
+        for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-                for (int db = 0; db < D / 32; db++) {
-                    bf16x8 a = lds_operand_tr(Vs, VS, kb * 16, db * 32, lane);
-                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
-                }
+            for (int r = 0; r < 16; r++) {
+                const float pv = __builtin_amdgcn_exp2f(s[nb][r] * c2 - mc);
+                s[nb][r] = pv;
+                psum += pv;
+            }
+        l_run += psum;
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
+            const bf16x8 pb = pack_bf16x8(s[kb >> 1], (kb & 1) * 8);
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) {
+                bf16x8 a = lds_operand_tr(Vs, VS, kb * 16, db * 32, lane);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
             }
         }
         have = have_next;
@@ -553,67 +568,153 @@ template <int D>
 struct BwdLds {
     static constexpr int BN = 128;      // keys per block, 32 per wave
     static constexpr int BM = 64;       // query rows per iteration (two 32-row MFMA sub-tiles)
-    static constexpr int QS = D + 8;    // Q / dO tile row stride (elements)
+    static constexpr int QS = D + 24;   // Q / dO tile row stride (elements): row + 48 B suits both the
+                                        // 128-bit operand reads and the transpose reads
     static constexpr int TILE = BM * QS;                                 // elements
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, lse, delta
     static constexpr int TOTAL = 2 * BUF_BYTES;
 };
 
-// One 32-row sub-tile for one wave (its 32 keys): S = Q K^T and dP = dO V^T by MFMA (query rows in
-// accumulator registers, this lane's key in the lane), P = exp2(S*c2 - LSE*log2e), dS = P*(dP - DELTA),
-// then dV^T += dO^T P and dK^T += Q^T dS with P / dS fed from registers as B operands and dO^T / Q^T
-// read from the same LDS tiles by transpose loads.
-template <int D, bool MASK>
-__device__ __forceinline__ void bwd_dkdv_sub_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s,
-                                                  const float *dlt_s, const bf16x8 (&kreg)[D / 16],
-                                                  const bf16x8 (&vreg)[D / 16], f32x16 (&dkacc)[D / 32],
-                                                  f32x16 (&dvacc)[D / 32], const f32x16 &zero16, int r0, int lane, int l32,
-                                                  int hh, float c2, bool key_ok, bool causal, int my_kpos, int row_base,
-                                                  int Sq, int q_split, int p0, int p1) {
+// Building blocks of one 64-row iteration of bwd_dkdv_kernel for one wave (its 32 keys).  A 32-row
+// sub-tile needs S = Q K^T and dP = dO V^T (query rows in accumulator registers, this lane's key in the
+// lane), then P = exp2(S*c2 - LSE*log2e) and dS = P*(dP - DELTA) element by element, then
+// dV^T += dO^T P and dK^T += Q^T dS with P / dS fed from registers as B operands and dO^T / Q^T read
+// from the same LDS tiles by transpose loads.  The softmax arithmetic of one sub-tile is issued between
+// the MFMAs of another (one element per MFMA) so the matrix pipe and the VALU run concurrently in a
+// single wave; sched_barrier keeps the compiler from regrouping the interleave.
+struct BwdMaskCtx {
+    bool key_ok, causal;
+    int my_kpos, row_base, Sq, q_split, p0, p1;
+};
+
+template <bool MASK>
+__device__ __forceinline__ void bwd_softmax_elem(f32x16 &s, f32x16 &dp, int r, float lse2, float dlt, float c2, int r0,
+                                                 int hh, const BwdMaskCtx &m) {
+    float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2);
+    float dsv = pv * (dp[r] - dlt);
+    if (MASK) {
+        const int qrow = m.row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
+        const int qpos = q_position(qrow, m.q_split, m.p0, m.p1);
+        const bool vis = m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
+        pv = vis ? pv : 0.f;
+        dsv = vis ? dsv : 0.f;
+    }
+    s[r] = pv;
+    dp[r] = dsv;
+}
+
+// S and dP of sub-tile r0 (16 MFMAs); when FUSE, the softmax arithmetic of the PREVIOUS sub-tile
+// (ps, pdp, rows pr0) rides along, one element per MFMA.
+template <int D, bool MASK, bool FUSE>
+__device__ __forceinline__ void bwd_gemm_s_dp(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
+                                              const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16], f32x16 &s,
+                                              f32x16 &dp, const f32x16 &zero16, int r0, int l32, int hh, f32x16 &ps,
+                                              f32x16 &pdp, int pr0, float c2, const BwdMaskCtx &m) {
     constexpr int QS = BwdLds<D>::QS;
-    f32x16 s = zero16, dp = zero16;
+    constexpr int NK = D / 16;
+    s = zero16;
+    dp = zero16;
+    const __bf16 *qrow = Qs + (r0 + l32) * QS + 8 * hh;
+    const __bf16 *drow = dOs + (r0 + l32) * QS + 8 * hh;
+    bf16x8 qa = *(const bf16x8 *)(qrow), da = *(const bf16x8 *)(drow);
+    f32x4 lv, dv;
 #pragma unroll
-    for (int kb = 0; kb < D / 16; kb++) {
-        bf16x8 a = *(const bf16x8 *)(Qs + (r0 + l32) * QS + kb * 16 + 8 * hh);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kreg[kb], s, 0, 0, 0);
+    for (int kb = 0; kb < NK; kb++) {
+        bf16x8 qn = qa, dn = da;
+        if (kb + 1 < NK) {
+            qn = *(const bf16x8 *)(qrow + (kb + 1) * 16);
+            dn = *(const bf16x8 *)(drow + (kb + 1) * 16);
+        }
+        if (FUSE && (2 * kb) % 4 == 0 && 2 * kb < 16) {
+            lv = *(const f32x4 *)(lse_s + pr0 + 8 * ((2 * kb) / 4) + 4 * hh);
+            dv = *(const f32x4 *)(dlt_s + pr0 + 8 * ((2 * kb) / 4) + 4 * hh);
+        }
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kreg[kb], s, 0, 0, 0);
+        if (FUSE && 2 * kb < 16) bwd_softmax_elem<MASK>(ps, pdp, 2 * kb, lv[(2 * kb) % 4], dv[(2 * kb) % 4], c2, pr0, hh, m);
+        __builtin_amdgcn_sched_barrier(0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vreg[kb], dp, 0, 0, 0);
+        if (FUSE && 2 * kb + 1 < 16)
+            bwd_softmax_elem<MASK>(ps, pdp, 2 * kb + 1, lv[(2 * kb + 1) % 4], dv[(2 * kb + 1) % 4], c2, pr0, hh, m);
+        __builtin_amdgcn_sched_barrier(0);
+        qa = qn;
+        da = dn;
     }
+    if (FUSE && 2 * NK < 16) {   // D = 64: only 8 MFMAs to hide behind; finish the rest here
 #pragma unroll
-    for (int kb = 0; kb < D / 16; kb++) {
-        bf16x8 a = *(const bf16x8 *)(dOs + (r0 + l32) * QS + kb * 16 + 8 * hh);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vreg[kb], dp, 0, 0, 0);
-    }
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const f32x4 lv = *(const f32x4 *)(lse_s + r0 + 8 * g + 4 * hh);
-        const f32x4 dv = *(const f32x4 *)(dlt_s + r0 + 8 * g + 4 * hh);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int r = 4 * g + e;
-            float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lv[e]);
-            float dsv = pv * (dp[r] - dv[e]);
-            if (MASK) {
-                const int qrow = row_base + r0 + 8 * g + 4 * hh + e;
-                const int qpos = q_position(qrow, q_split, p0, p1);
-                const bool vis = key_ok && qrow < Sq && (!causal || my_kpos <= qpos);
-                pv = vis ? pv : 0.f;
-                dsv = vis ? dsv : 0.f;
+        for (int r = 2 * NK; r < 16; r++) {
+            if (r % 4 == 0) {
+                lv = *(const f32x4 *)(lse_s + pr0 + 8 * (r / 4) + 4 * hh);
+                dv = *(const f32x4 *)(dlt_s + pr0 + 8 * (r / 4) + 4 * hh);
             }
-            s[r] = pv;
-            dp[r] = dsv;
+            bwd_softmax_elem<MASK>(ps, pdp, r, lv[r % 4], dv[r % 4], c2, pr0, hh, m);
         }
     }
+}
+
+// dV^T += dO^T P and dK^T += Q^T dS of sub-tile r0 (16 MFMAs for D = 128); when FUSE, the softmax
+// arithmetic of the NEXT sub-tile (ns, ndp, rows nr0) rides along.
+template <int D, bool MASK, bool FUSE>
+__device__ __forceinline__ void bwd_gemm_dv_dk(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
+                                               f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &s,
+                                               const f32x16 &dp, int r0, int lane, int hh, f32x16 &ns, f32x16 &ndp, int nr0,
+                                               float c2, const BwdMaskCtx &m) {
+    constexpr int QS = BwdLds<D>::QS;
+    constexpr int ND = D / 32;
+    f32x4 lv, dv;
+    bf16x8 ao = lds_operand_tr(dOs, QS, r0, 0, lane), aq = lds_operand_tr(Qs, QS, r0, 0, lane);
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
-        bf16x8 pb = pack_bf16x8(s, kb * 8);
-        bf16x8 dsb = pack_bf16x8(dp, kb * 8);
+        const bf16x8 pb = pack_bf16x8(s, kb * 8);
+        const bf16x8 dsb = pack_bf16x8(dp, kb * 8);
 #pragma unroll
-        for (int db = 0; db < D / 32; db++) {
-            bf16x8 a = lds_operand_tr(dOs, QS, r0 + kb * 16, db * 32, lane);
-            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, dvacc[db], 0, 0, 0);
-            bf16x8 a2 = lds_operand_tr(Qs, QS, r0 + kb * 16, db * 32, lane);
-            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, dsb, dkacc[db], 0, 0, 0);
+        for (int db = 0; db < ND; db++) {
+            const int step = kb * ND + db;              // 0 .. 2*ND-1, two MFMAs per step
+            bf16x8 aon = ao, aqn = aq;
+            if (step + 1 < 2 * ND) {
+                const int nkb = (step + 1) / ND, ndb = (step + 1) % ND;
+                aon = lds_operand_tr(dOs, QS, r0 + nkb * 16, ndb * 32, lane);
+                aqn = lds_operand_tr(Qs, QS, r0 + nkb * 16, ndb * 32, lane);
+            }
+            constexpr int EPS = 16 / (2 * ND);          // softmax elements per step (2 for D=128, 4 for D=64)
+            if (FUSE && (step * EPS) % 4 == 0) {
+                lv = *(const f32x4 *)(lse_s + nr0 + 8 * ((step * EPS) / 4) + 4 * hh);
+                dv = *(const f32x4 *)(dlt_s + nr0 + 8 * ((step * EPS) / 4) + 4 * hh);
+            }
+            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pb, dvacc[db], 0, 0, 0);
+            if (FUSE) {
+#pragma unroll
+                for (int e = 0; e < EPS / 2; e++) {
+                    const int r = step * EPS + e;
+                    bwd_softmax_elem<MASK>(ns, ndp, r, lv[r % 4], dv[r % 4], c2, nr0, hh, m);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsb, dkacc[db], 0, 0, 0);
+            if (FUSE) {
+#pragma unroll
+                for (int e = EPS / 2; e < EPS; e++) {
+                    const int r = step * EPS + e;
+                    bwd_softmax_elem<MASK>(ns, ndp, r, lv[r % 4], dv[r % 4], c2, nr0, hh, m);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            ao = aon;
+            aq = aqn;
         }
     }
+}
+
+// One 64-row tile (sub-tiles a = rows 0..31, b = rows 32..63) for one wave.
+template <int D, bool MASK>
+__device__ __forceinline__ void bwd_dkdv_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
+                                              const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16],
+                                              f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &zero16,
+                                              int lane, int l32, int hh, float c2, const BwdMaskCtx &m) {
+    f32x16 sa, dpa, sb, dpb;
+    bwd_gemm_s_dp<D, MASK, false>(Qs, dOs, lse_s, dlt_s, kreg, vreg, sa, dpa, zero16, 0, l32, hh, sa, dpa, 0, c2, m);
+    bwd_gemm_s_dp<D, MASK, true>(Qs, dOs, lse_s, dlt_s, kreg, vreg, sb, dpb, zero16, 32, l32, hh, sa, dpa, 0, c2, m);
+    bwd_gemm_dv_dk<D, MASK, true>(Qs, dOs, lse_s, dlt_s, dkacc, dvacc, sa, dpa, 0, lane, hh, sb, dpb, 32, c2, m);
+    bwd_gemm_dv_dk<D, MASK, false>(Qs, dOs, lse_s, dlt_s, dkacc, dvacc, sb, dpb, 32, lane, hh, sb, dpb, 32, c2, m);
 }
 
 template <int D>
@@ -688,11 +789,11 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     }
     const float c2 = p.scale * LTR_LOG2E;
 
-    // iteration space: (query head of the group, 64-row query tile).  Class 0: no row sees any key of
-    // the block (skipped); 1: every (row, key) pair is visible; 2: needs the mask (diagonal, tails).
-    const int n_it = p.n_rep * p.n_qtiles;
-    auto tile_class = [&](int it) {
-        const int row0 = (it % p.n_qtiles) * BM;
+    // iteration space: (query head of the group, 64-row query tile).  A tile's class depends on its
+    // rows only: 0 = no row sees any key of the block (skipped); 1 = every (row, key) pair is visible;
+    // 2 = needs the mask (diagonal, tails).
+    auto tile_class = [&](int qt) {
+        const int row0 = qt * BM;
         const bool edge = key_tail || row0 + BM > p.Sq;
         if (!causal) return edge ? 2 : 1;
         int lo, hi;
@@ -700,87 +801,107 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         if (hi < tile_kpos_lo) return 0;
         return (edge || tile_kpos_hi > lo) ? 2 : 1;
     };
-    auto next_of = [&](int it, int cls) {
-        while (it < n_it && tile_class(it) != cls) it++;
-        return it;
-    };
 
     // per-thread staging coordinates: row (tid / CPR) + RPL*i, 16-byte chunk tid % CPR
     const int ld_r = tid / CPR, ld_c = tid % CPR;
     const unsigned q_voff = (unsigned)(ld_r * (int)p.qs[1] + ld_c * 8);
     const unsigned do_voff = (unsigned)(ld_r * (int)p.dos[1] + ld_c * 8);
+    const float st_mul = tid < BM ? LTR_LOG2E : 1.f;  // threads 0..63 stage LSE*log2e, 64..127 stage DELTA
     uint4 qld[NLD], dld[NLD];
-    float sld = 0.f;  // threads 0..63: LSE*log2e of row tid; threads 64..127: DELTA of row tid-64
-    auto gload = [&](int it) {
-        const int h = hkv * p.n_rep + it / p.n_qtiles;
-        const int row0 = (it % p.n_qtiles) * BM;
-        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2] + (long long)row0 * p.qs[1];
-        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2] + (long long)row0 * p.dos[1];
-        const float *lsep = p.lse + ((long long)b * p.Hq + h) * p.Sq + row0;
-        const float *dltp = p.delta + ((long long)b * p.Hq + h) * p.Sq + row0;
-        if (row0 + BM <= p.Sq) {
-#pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                qld[i] = *(const uint4 *)(qp + (q_voff + (unsigned)(i * RPL * (int)p.qs[1])));
-                dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
-            }
-            if (tid < BM) sld = lsep[tid] * LTR_LOG2E;
-            else if (tid < 2 * BM) sld = dltp[tid - BM];
-        } else {
-#pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                qld[i] = make_uint4(0, 0, 0, 0);
-                dld[i] = make_uint4(0, 0, 0, 0);
-                if (row0 + ld_r + i * RPL < p.Sq) {
-                    qld[i] = *(const uint4 *)(qp + (q_voff + (unsigned)(i * RPL * (int)p.qs[1])));
-                    dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
-                }
-            }
-            // rows past the end: LSE = +inf makes P = 0 (they are masked as well)
-            if (tid < BM) sld = (row0 + tid < p.Sq) ? lsep[tid] * LTR_LOG2E : INFINITY;
-            else if (tid < 2 * BM) sld = (row0 + tid - BM < p.Sq) ? dltp[tid - BM] : 0.f;
-        }
-    };
-    auto lds_store = [&](int buf) {
-        __bf16 *Qs = (__bf16 *)(smem + buf * L::BUF_BYTES);
-        __bf16 *dOs = Qs + L::TILE;
-        float *st = (float *)(dOs + L::TILE);
-#pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            *(uint4 *)(Qs + (ld_r + i * RPL) * QS + ld_c * 8) = qld[i];
-            *(uint4 *)(dOs + (ld_r + i * RPL) * QS + ld_c * 8) = dld[i];
-        }
-        if (tid < 2 * BM) st[tid] = sld;
-    };
+    float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
+    bool sld_ok = true;
 
     // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
-    // live in straight-line loop bodies
+    // live in straight-line loop bodies and the unmasked pass carries no bounds checks at all
     auto run_pass = [&](auto mask_tag) {
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr int cls = MASK ? 2 : 1;
-        int it = next_of(0, cls);
-        if (it >= n_it) return;
+        auto advance = [&](int &rep, int &qt) {   // next tile of this class after (rep, qt); false when done
+            for (;;) {
+                if (++qt >= p.n_qtiles) {
+                    qt = 0;
+                    if (++rep >= p.n_rep) return false;
+                }
+                if (tile_class(qt) == cls) return true;
+            }
+        };
+        auto gload = [&](int rep, int qt) {
+            const int h = hkv * p.n_rep + rep;
+            const int row0 = qt * BM;
+            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2] + (long long)row0 * p.qs[1];
+            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2] + (long long)row0 * p.dos[1];
+            const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
+            const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
+            if (!MASK) {
+#pragma unroll
+                for (int i = 0; i < NLD; i++) {
+                    qld[i] = *(const uint4 *)(qp + (q_voff + (unsigned)(i * RPL * (int)p.qs[1])));
+                    dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
+                }
+                if (tid < 2 * BM) sld = sp[tid];
+            } else {
+#pragma unroll
+                for (int i = 0; i < NLD; i++) {
+                    const bool ok = row0 + ld_r + i * RPL < p.Sq;
+                    const unsigned qo = ok ? q_voff + (unsigned)(i * RPL * (int)p.qs[1]) : 0u;
+                    const unsigned dO = ok ? do_voff + (unsigned)(i * RPL * (int)p.dos[1]) : 0u;
+                    qld[i] = *(const uint4 *)(qp + qo);     // row0 itself is always a valid row
+                    dld[i] = *(const uint4 *)(dop + dO);
+                    if (!ok) {
+                        qld[i] = make_uint4(0, 0, 0, 0);
+                        dld[i] = make_uint4(0, 0, 0, 0);
+                    }
+                }
+                if (tid < 2 * BM) {
+                    const int r = tid < BM ? tid : tid - BM;
+                    sld_ok = row0 + r < p.Sq;
+                    sld = sp[sld_ok ? tid : (tid < BM ? 0 : BM)];
+                }
+            }
+        };
+        auto lds_store = [&](int buf) {
+            __bf16 *Qs = (__bf16 *)(smem + buf * L::BUF_BYTES);
+            __bf16 *dOs = Qs + L::TILE;
+            float *st = (float *)(dOs + L::TILE);
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                *(uint4 *)(Qs + (ld_r + i * RPL) * QS + ld_c * 8) = qld[i];
+                *(uint4 *)(dOs + (ld_r + i * RPL) * QS + ld_c * 8) = dld[i];
+            }
+            if (tid < 2 * BM) {
+                float x = sld * st_mul;
+                // rows past the end: LSE = +inf makes P = 0 (they are masked as well)
+                if (MASK) x = sld_ok ? x : (tid < BM ? INFINITY : 0.f);
+                st[tid] = x;
+            }
+        };
+
+        BwdMaskCtx mctx;
+        mctx.key_ok = key_ok;
+        mctx.causal = causal;
+        mctx.my_kpos = my_kpos;
+        mctx.Sq = p.Sq;
+        mctx.q_split = p.q_split;
+        mctx.p0 = p.q_pos0[0];
+        mctx.p1 = p.q_pos0[1];
+        int rep = 0, qt = -1;
+        if (!advance(rep, qt)) return;
         __syncthreads();   // the previous pass has finished reading LDS
-        gload(it);
+        gload(rep, qt);
         lds_store(0);
         __syncthreads();
         int par = 0;
-        while (it < n_it) {
-            const int it_next = next_of(it + 1, cls);
-            if (it_next < n_it) gload(it_next);
-            const int row0 = (it % p.n_qtiles) * BM;
+        for (bool more = true; more;) {
+            mctx.row_base = qt * BM;
+            more = advance(rep, qt);
+            if (more) gload(rep, qt);
             const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
             const __bf16 *dOs = Qs + L::TILE;
             const float *lse_s = (const float *)(dOs + L::TILE);
             const float *dlt_s = lse_s + BM;
-#pragma unroll
-            for (int sub = 0; sub < 2; sub++)
-                bwd_dkdv_sub_tile<D, MASK>(Qs, dOs, lse_s, dlt_s, kreg, vreg, dkacc, dvacc, zero16, sub * 32, lane, l32,
-                                           hh, c2, key_ok, causal, my_kpos, row0, p.Sq, p.q_split, p.q_pos0[0],
-                                           p.q_pos0[1]);
-            if (it_next < n_it) lds_store(par ^ 1);
+            bwd_dkdv_tile<D, MASK>(Qs, dOs, lse_s, dlt_s, kreg, vreg, dkacc, dvacc, zero16, lane, l32, hh, c2, mctx);
+            if (more) lds_store(par ^ 1);
             __syncthreads();
-            it = it_next;
             par ^= 1;
         }
     };
@@ -814,8 +935,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 template <int D>
 __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdParams p) {
     constexpr int BM = 128, BN = 64;
-    constexpr int KS = D + 8;
-    constexpr int VS = D + 8;
+    constexpr int KS = D + 24;   // K tile: 128-bit operand reads and transpose reads (row + 48 B)
+    constexpr int VS = D + 8;    // V tile: 128-bit operand reads only (row + 16 B)
     constexpr int CPR = D / 8;
     constexpr int NLD = BN * CPR / 256;
     __shared__ __attribute__((aligned(16))) __bf16 Ks[BN * KS];
