@@ -12,6 +12,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-shared", "-fPIC", "-std=c++17",
     "-munsafe-fp-atomics",                      # hardware global_atomic_add_f32 for the dQ accumulator
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",       # MFMA results in VGPRs: no accvgpr copies around the softmax
     "-I", os.path.join(ROOT, "include"),
 ]
 

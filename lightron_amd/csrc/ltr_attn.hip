@@ -30,6 +30,7 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
@@ -575,146 +576,202 @@ struct BwdLds {
     static constexpr int TOTAL = 2 * BUF_BYTES;
 };
 
-// Building blocks of one 64-row iteration of bwd_dkdv_kernel for one wave (its 32 keys).  A 32-row
-// sub-tile needs S = Q K^T and dP = dO V^T (query rows in accumulator registers, this lane's key in the
-// lane), then P = exp2(S*c2 - LSE*log2e) and dS = P*(dP - DELTA) element by element, then
+// One 64-row iteration of bwd_dkdv_kernel for one wave (its 32 keys), as two 32-row sub-tiles a, b.
+// A sub-tile needs S = Q K^T and dP = dO V^T (query rows in accumulator registers, this lane's key in
+// the lane), then P = exp2(S*c2 - LSE*log2e) and dS = P*(dP - DELTA) element by element, then
 // dV^T += dO^T P and dK^T += Q^T dS with P / dS fed from registers as B operands and dO^T / Q^T read
-// from the same LDS tiles by transpose loads.  The softmax arithmetic of one sub-tile is issued between
-// the MFMAs of another (one element per MFMA) so the matrix pipe and the VALU run concurrently in a
-// single wave; sched_barrier keeps the compiler from regrouping the interleave.
+// from the same LDS tiles by transpose loads.  Order of issue:
+//     S_a, dP_a | S_b, dP_b + softmax(a) | dV, dK (a) + softmax(b) | dV, dK (b)
+// so the softmax arithmetic of one sub-tile sits between the MFMAs of another and the matrix pipe and
+// the VALU run concurrently inside a single wave; sched_barrier keeps the interleave.  MFMA results are
+// read once and P / dS go straight to packed bf16 pairs (never written back to the accumulator tile).
 struct BwdMaskCtx {
     bool key_ok, causal;
     int my_kpos, row_base, Sq, q_split, p0, p1;
 };
 
+struct PackedTile {   // 16 bf16 values of one lane's 32x32 tile column, as the two B operands of K = 16
+    unsigned u[8];
+};
+
+__device__ __forceinline__ unsigned pack2_bf16(float a, float b) {
+    bf16x2 t;
+    t[0] = (__bf16)a;
+    t[1] = (__bf16)b;
+    return __builtin_bit_cast(unsigned, t);
+}
+
+__device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
+    union { unsigned u[4]; bf16x8 v; } c;
+    c.u[0] = t.u[4 * kb];
+    c.u[1] = t.u[4 * kb + 1];
+    c.u[2] = t.u[4 * kb + 2];
+    c.u[3] = t.u[4 * kb + 3];
+    return c.v;
+}
+
+// elements 2j and 2j+1 of a sub-tile: P and dS pairs
 template <bool MASK>
-__device__ __forceinline__ void bwd_softmax_elem(f32x16 &s, f32x16 &dp, int r, float lse2, float dlt, float c2, int r0,
-                                                 int hh, const BwdMaskCtx &m) {
-    float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2);
-    float dsv = pv * (dp[r] - dlt);
-    if (MASK) {
-        const int qrow = m.row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
-        const int qpos = q_position(qrow, m.q_split, m.p0, m.p1);
-        const bool vis = m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
-        pv = vis ? pv : 0.f;
-        dsv = vis ? dsv : 0.f;
+__device__ __forceinline__ void bwd_softmax_pair(const f32x16 &s, const f32x16 &dp, int j, const f32x4 &lv, const f32x4 &dv,
+                                                 float c2, int r0, int hh, const BwdMaskCtx &m, PackedTile &pp,
+                                                 PackedTile &pds) {
+    float pv[2], dsv[2];
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        const int r = 2 * j + e;
+        pv[e] = __builtin_amdgcn_exp2f(s[r] * c2 - lv[r % 4]);
+        dsv[e] = pv[e] * (dp[r] - dv[r % 4]);
+        if (MASK) {
+            const int qrow = m.row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
+            const int qpos = q_position(qrow, m.q_split, m.p0, m.p1);
+            const bool vis = m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
+            pv[e] = vis ? pv[e] : 0.f;
+            dsv[e] = vis ? dsv[e] : 0.f;
+        }
     }
-    s[r] = pv;
-    dp[r] = dsv;
+    pp.u[j] = pack2_bf16(pv[0], pv[1]);
+    pds.u[j] = pack2_bf16(dsv[0], dsv[1]);
 }
 
-// S and dP of sub-tile r0 (16 MFMAs); when FUSE, the softmax arithmetic of the PREVIOUS sub-tile
-// (ps, pdp, rows pr0) rides along, one element per MFMA.
-template <int D, bool MASK, bool FUSE>
-__device__ __forceinline__ void bwd_gemm_s_dp(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
-                                              const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16], f32x16 &s,
-                                              f32x16 &dp, const f32x16 &zero16, int r0, int l32, int hh, f32x16 &ps,
-                                              f32x16 &pdp, int pr0, float c2, const BwdMaskCtx &m) {
-    constexpr int QS = BwdLds<D>::QS;
-    constexpr int NK = D / 16;
-    s = zero16;
-    dp = zero16;
-    const __bf16 *qrow = Qs + (r0 + l32) * QS + 8 * hh;
-    const __bf16 *drow = dOs + (r0 + l32) * QS + 8 * hh;
-    bf16x8 qa = *(const bf16x8 *)(qrow), da = *(const bf16x8 *)(drow);
-    f32x4 lv, dv;
-#pragma unroll
-    for (int kb = 0; kb < NK; kb++) {
-        bf16x8 qn = qa, dn = da;
-        if (kb + 1 < NK) {
-            qn = *(const bf16x8 *)(qrow + (kb + 1) * 16);
-            dn = *(const bf16x8 *)(drow + (kb + 1) * 16);
-        }
-        if (FUSE && (2 * kb) % 4 == 0 && 2 * kb < 16) {
-            lv = *(const f32x4 *)(lse_s + pr0 + 8 * ((2 * kb) / 4) + 4 * hh);
-            dv = *(const f32x4 *)(dlt_s + pr0 + 8 * ((2 * kb) / 4) + 4 * hh);
-        }
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kreg[kb], s, 0, 0, 0);
-        if (FUSE && 2 * kb < 16) bwd_softmax_elem<MASK>(ps, pdp, 2 * kb, lv[(2 * kb) % 4], dv[(2 * kb) % 4], c2, pr0, hh, m);
-        __builtin_amdgcn_sched_barrier(0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vreg[kb], dp, 0, 0, 0);
-        if (FUSE && 2 * kb + 1 < 16)
-            bwd_softmax_elem<MASK>(ps, pdp, 2 * kb + 1, lv[(2 * kb + 1) % 4], dv[(2 * kb + 1) % 4], c2, pr0, hh, m);
-        __builtin_amdgcn_sched_barrier(0);
-        qa = qn;
-        da = dn;
-    }
-    if (FUSE && 2 * NK < 16) {   // D = 64: only 8 MFMAs to hide behind; finish the rest here
-#pragma unroll
-        for (int r = 2 * NK; r < 16; r++) {
-            if (r % 4 == 0) {
-                lv = *(const f32x4 *)(lse_s + pr0 + 8 * (r / 4) + 4 * hh);
-                dv = *(const f32x4 *)(dlt_s + pr0 + 8 * (r / 4) + 4 * hh);
-            }
-            bwd_softmax_elem<MASK>(ps, pdp, r, lv[r % 4], dv[r % 4], c2, pr0, hh, m);
-        }
-    }
-}
-
-// dV^T += dO^T P and dK^T += Q^T dS of sub-tile r0 (16 MFMAs for D = 128); when FUSE, the softmax
-// arithmetic of the NEXT sub-tile (ns, ndp, rows nr0) rides along.
-template <int D, bool MASK, bool FUSE>
-__device__ __forceinline__ void bwd_gemm_dv_dk(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
-                                               f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &s,
-                                               const f32x16 &dp, int r0, int lane, int hh, f32x16 &ns, f32x16 &ndp, int nr0,
-                                               float c2, const BwdMaskCtx &m) {
-    constexpr int QS = BwdLds<D>::QS;
-    constexpr int ND = D / 32;
-    f32x4 lv, dv;
-    bf16x8 ao = lds_operand_tr(dOs, QS, r0, 0, lane), aq = lds_operand_tr(Qs, QS, r0, 0, lane);
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-        const bf16x8 pb = pack_bf16x8(s, kb * 8);
-        const bf16x8 dsb = pack_bf16x8(dp, kb * 8);
-#pragma unroll
-        for (int db = 0; db < ND; db++) {
-            const int step = kb * ND + db;              // 0 .. 2*ND-1, two MFMAs per step
-            bf16x8 aon = ao, aqn = aq;
-            if (step + 1 < 2 * ND) {
-                const int nkb = (step + 1) / ND, ndb = (step + 1) % ND;
-                aon = lds_operand_tr(dOs, QS, r0 + nkb * 16, ndb * 32, lane);
-                aqn = lds_operand_tr(Qs, QS, r0 + nkb * 16, ndb * 32, lane);
-            }
-            constexpr int EPS = 16 / (2 * ND);          // softmax elements per step (2 for D=128, 4 for D=64)
-            if (FUSE && (step * EPS) % 4 == 0) {
-                lv = *(const f32x4 *)(lse_s + nr0 + 8 * ((step * EPS) / 4) + 4 * hh);
-                dv = *(const f32x4 *)(dlt_s + nr0 + 8 * ((step * EPS) / 4) + 4 * hh);
-            }
-            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pb, dvacc[db], 0, 0, 0);
-            if (FUSE) {
-#pragma unroll
-                for (int e = 0; e < EPS / 2; e++) {
-                    const int r = step * EPS + e;
-                    bwd_softmax_elem<MASK>(ns, ndp, r, lv[r % 4], dv[r % 4], c2, nr0, hh, m);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsb, dkacc[db], 0, 0, 0);
-            if (FUSE) {
-#pragma unroll
-                for (int e = EPS / 2; e < EPS; e++) {
-                    const int r = step * EPS + e;
-                    bwd_softmax_elem<MASK>(ns, ndp, r, lv[r % 4], dv[r % 4], c2, nr0, hh, m);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            ao = aon;
-            aq = aqn;
-        }
-    }
-}
-
-// One 64-row tile (sub-tiles a = rows 0..31, b = rows 32..63) for one wave.
 template <int D, bool MASK>
 __device__ __forceinline__ void bwd_dkdv_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
                                               const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16],
                                               f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &zero16,
                                               int lane, int l32, int hh, float c2, const BwdMaskCtx &m) {
-    f32x16 sa, dpa, sb, dpb;
-    bwd_gemm_s_dp<D, MASK, false>(Qs, dOs, lse_s, dlt_s, kreg, vreg, sa, dpa, zero16, 0, l32, hh, sa, dpa, 0, c2, m);
-    bwd_gemm_s_dp<D, MASK, true>(Qs, dOs, lse_s, dlt_s, kreg, vreg, sb, dpb, zero16, 32, l32, hh, sa, dpa, 0, c2, m);
-    bwd_gemm_dv_dk<D, MASK, true>(Qs, dOs, lse_s, dlt_s, dkacc, dvacc, sa, dpa, 0, lane, hh, sb, dpb, 32, c2, m);
-    bwd_gemm_dv_dk<D, MASK, false>(Qs, dOs, lse_s, dlt_s, dkacc, dvacc, sb, dpb, 32, lane, hh, sb, dpb, 32, c2, m);
+    constexpr int QS = BwdLds<D>::QS;
+    constexpr int NK = D / 16, ND = D / 32;
+    f32x16 sa = zero16, dpa = zero16, sb = zero16, dpb = zero16;
+    PackedTile pa, dsa, pb, dsb;
+    const __bf16 *qrow = Qs + l32 * QS + 8 * hh;
+    const __bf16 *drow = dOs + l32 * QS + 8 * hh;
+    const float *lrow = lse_s + 4 * hh, *trow = dlt_s + 4 * hh;
+
+    // S_a, dP_a (operands fetched two steps ahead of their MFMAs)
+    {
+        bf16x8 qb[3], db_[3];
+        qb[0] = *(const bf16x8 *)(qrow);
+        db_[0] = *(const bf16x8 *)(drow);
+        qb[1] = *(const bf16x8 *)(qrow + 16);
+        db_[1] = *(const bf16x8 *)(drow + 16);
+#pragma unroll
+        for (int kb = 0; kb < NK; kb++) {
+            if (kb + 2 < NK) {
+                qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + (kb + 2) * 16);
+                db_[(kb + 2) % 3] = *(const bf16x8 *)(drow + (kb + 2) * 16);
+            }
+            sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], sa, 0, 0, 0);
+            dpa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db_[kb % 3], vreg[kb], dpa, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // S_b, dP_b with softmax(a): 8 pairs over 2*NK MFMAs
+    {
+        f32x4 lv = *(const f32x4 *)(lrow), dv = *(const f32x4 *)(trow);
+        bf16x8 qb[3], db_[3];
+        qb[0] = *(const bf16x8 *)(qrow + 32 * QS);
+        db_[0] = *(const bf16x8 *)(drow + 32 * QS);
+        qb[1] = *(const bf16x8 *)(qrow + 32 * QS + 16);
+        db_[1] = *(const bf16x8 *)(drow + 32 * QS + 16);
+#pragma unroll
+        for (int kb = 0; kb < NK; kb++) {
+            constexpr int PPS = 8 / NK > 0 ? 8 / NK : 1;    // pairs per kb step (1 for D=128, 2 for D=64)
+            if (kb + 2 < NK) {
+                qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + 32 * QS + (kb + 2) * 16);
+                db_[(kb + 2) % 3] = *(const bf16x8 *)(drow + 32 * QS + (kb + 2) * 16);
+            }
+            f32x4 lvn = lv, dvn = dv;
+            {
+                const int jn = (kb + 1) * PPS;              // first pair of the next step
+                if (jn < 8 && jn % 2 == 0) {
+                    lvn = *(const f32x4 *)(lrow + 8 * (jn / 2));
+                    dvn = *(const f32x4 *)(trow + 8 * (jn / 2));
+                }
+            }
+            sb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], sb, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < PPS; q++) {
+                const int j = kb * PPS + q;
+                if (j < 8) {
+                    if (q > 0 && j % 2 == 0) {              // D = 64: a new row group inside the step
+                        lv = *(const f32x4 *)(lrow + 8 * (j / 2));
+                        dv = *(const f32x4 *)(trow + 8 * (j / 2));
+                    }
+                    bwd_softmax_pair<MASK>(sa, dpa, j, lv, dv, c2, 0, hh, m, pa, dsa);
+                }
+            }
+            dpb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db_[kb % 3], vreg[kb], dpb, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            lv = lvn;
+            dv = dvn;
+        }
+    }
+    // dV, dK of sub-tile a with softmax(b): 8 pairs over 2*ND steps of two MFMAs
+    {
+        f32x4 lv = *(const f32x4 *)(lrow + 32), dv = *(const f32x4 *)(trow + 32);
+        bf16x8 ao = lds_operand_tr(dOs, QS, 0, 0, lane), aq = lds_operand_tr(Qs, QS, 0, 0, lane);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const bf16x8 pop = operand_of(pa, kb), dsop = operand_of(dsa, kb);
+#pragma unroll
+            for (int db = 0; db < ND; db++) {
+                const int step = kb * ND + db;
+                constexpr int PPS = 8 / (2 * ND);           // pairs per step (1 for D=128, 2 for D=64)
+                bf16x8 aon = ao, aqn = aq;
+                if (step + 1 < 2 * ND) {
+                    const int nkb = (step + 1) / ND, ndb = (step + 1) % ND;
+                    aon = lds_operand_tr(dOs, QS, nkb * 16, ndb * 32, lane);
+                    aqn = lds_operand_tr(Qs, QS, nkb * 16, ndb * 32, lane);
+                } else {                                    // first operands of the sub-tile b phase
+                    aon = lds_operand_tr(dOs, QS, 32, 0, lane);
+                    aqn = lds_operand_tr(Qs, QS, 32, 0, lane);
+                }
+                f32x4 lvn = lv, dvn = dv;
+                {
+                    const int jn = (step + 1) * PPS;
+                    if (jn < 8 && jn % 2 == 0) {
+                        lvn = *(const f32x4 *)(lrow + 32 + 8 * (jn / 2));
+                        dvn = *(const f32x4 *)(trow + 32 + 8 * (jn / 2));
+                    }
+                }
+                dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pop, dvacc[db], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < PPS; q++) {
+                    const int j = step * PPS + q;
+                    if (q > 0 && j % 2 == 0) {
+                        lv = *(const f32x4 *)(lrow + 32 + 8 * (j / 2));
+                        dv = *(const f32x4 *)(trow + 32 + 8 * (j / 2));
+                    }
+                    bwd_softmax_pair<MASK>(sb, dpb, j, lv, dv, c2, 32, hh, m, pb, dsb);
+                }
+                dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsop, dkacc[db], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                ao = aon;
+                aq = aqn;
+                lv = lvn;
+                dv = dvn;
+            }
+        }
+        // dV, dK of sub-tile b
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const bf16x8 pop = operand_of(pb, kb), dsop = operand_of(dsb, kb);
+#pragma unroll
+            for (int db = 0; db < ND; db++) {
+                const int step = kb * ND + db;
+                bf16x8 aon = ao, aqn = aq;
+                if (step + 1 < 2 * ND) {
+                    const int nkb = (step + 1) / ND, ndb = (step + 1) % ND;
+                    aon = lds_operand_tr(dOs, QS, 32 + nkb * 16, ndb * 32, lane);
+                    aqn = lds_operand_tr(Qs, QS, 32 + nkb * 16, ndb * 32, lane);
+                }
+                dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pop, dvacc[db], 0, 0, 0);
+                dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsop, dkacc[db], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                ao = aon;
+                aq = aqn;
+            }
+        }
+    }
 }
 
 template <int D>
