@@ -163,28 +163,35 @@ def main():
                 out.append(acc[j])
         return out
 
-    ev = {"fwd": [], "bwd": []}
+    ev = {"fwd": [], "dkdv": [], "dq": []}
+
+    def timed_call(key, timed, fn):
+        if not timed:
+            return fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        r = fn()
+        e1.record()
+        ev[key].append((e0, e1))
+        return r
 
     def step(timed):
         if bwd:
             dq_acc.zero_(); dk_acc.zero_(); dv_acc.zero_()
         for r in cfg["ranks"]:
             ks, vs, pos, qp, qsplit = tables[r]
-            if timed:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            la.attn_fwd(q_all[r], ks, vs, pos, qp, qsplit, causal, out=o_all[r], lse=lse_all[r])
-            if timed:
-                e1.record(); ev["fwd"].append((e0, e1))
+            timed_call("fwd", timed, lambda: la.attn_fwd(q_all[r], ks, vs, pos, qp, qsplit, causal, out=o_all[r],
+                                                         lse=lse_all[r]))
             if bwd:
                 delta = la.attn_delta(o_all[r], do_all[r])
-                if timed:
-                    e2, e3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e2.record()
-                la.attn_bwd_accumulate(q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_acc[r],
-                                       acc_views(r, dk_acc), acc_views(r, dv_acc), qp, qsplit, causal)
-                if timed:
-                    e3.record(); ev["bwd"].append((e2, e3))
+                dks, dvs = acc_views(r, dk_acc), acc_views(r, dv_acc)
+                # the two backward kernels are enqueued by two calls so each can be timed on its own
+                timed_call("dkdv", timed, lambda: la.attn_bwd_accumulate(
+                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_acc[r], dks, dvs, qp, qsplit, causal,
+                    do_dq=False))
+                timed_call("dq", timed, lambda: la.attn_bwd_accumulate(
+                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_acc[r], dks, dvs, qp, qsplit, causal,
+                    do_dkdv=False))
         if bwd:
             la.cast_to_bf16(dq_acc); la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
 
@@ -201,14 +208,23 @@ def main():
     f_fwd = 4.0 * B * Hq * D * pairs
     f_total = f_fwd * (3.5 if bwd else 1.0)
     tflops = f_total / dt / 1e12
-    fwd_ms = sum(a.elapsed_time(b) for a, b in ev["fwd"]) / len(ev["fwd"])
+    avg = lambda key: sum(a.elapsed_time(b) for a, b in ev[key]) / len(ev[key])
+    fwd_ms = avg("fwd")
     launches = len(cfg["ranks"])
+    f_share = f_fwd / launches                      # forward flops of one launch (one rank's share)
+    kernels = {"fwd_bf16_kernel": {"ms_per_launch": round(fwd_ms, 4), "algorithmic_tflops": round(f_share / fwd_ms / 1e9, 2),
+                                   "gemms_credited": 2, "gemms_executed": 2}}
     if bwd:
-        bwd_ms = sum(a.elapsed_time(b) for a, b in ev["bwd"]) / len(ev["bwd"])
-        dom, dom_ms, dom_flops = "bwd_bf16_kernel<%d>" % D, bwd_ms, 2.5 * f_fwd / launches
+        # credited backward work is 5 GEMMs (S, dP, dV, dK, dQ); the dQ kernel recomputes S and dP
+        dkdv_ms, dq_ms = avg("dkdv"), avg("dq")
+        kernels["bwd_dkdv_kernel"] = {"ms_per_launch": round(dkdv_ms, 4), "gemms_credited": 4, "gemms_executed": 4,
+                                      "algorithmic_tflops": round(2.0 * f_share / dkdv_ms / 1e9, 2)}
+        kernels["bwd_dq_kernel"] = {"ms_per_launch": round(dq_ms, 4), "gemms_credited": 1, "gemms_executed": 3,
+                                    "algorithmic_tflops": round(0.5 * f_share / dq_ms / 1e9, 2),
+                                    "executed_tflops": round(1.5 * f_share / dq_ms / 1e9, 2)}
+        dom, dom_ms, dom_flops = "bwd_dkdv_kernel<%d>" % D, dkdv_ms, 2.0 * f_share
     else:
-        bwd_ms = None
-        dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_fwd / launches
+        dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_share
     achieved = dom_flops / (dom_ms * 1e-3) / 1e12
     prop = torch.cuda.get_device_properties(0)
     out = {
@@ -219,10 +235,7 @@ def main():
         "config": {"workload": cfg["desc"], "B": B, "Hq": Hq, "Hkv": Hkv, "D": D, "S": S, "ranks": launches,
                    "layout": cfg["layout"], "causal": causal, "flops_per_step": f_total},
         "frac_of_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        "kernels": {"fwd_ms_per_launch": round(fwd_ms, 4),
-                    "fwd_tflops": round(f_fwd / launches / (fwd_ms * 1e-3) / 1e12, 2),
-                    "bwd_ms_per_launch": None if bwd_ms is None else round(bwd_ms, 4),
-                    "bwd_tflops": None if bwd_ms is None else round(2.5 * f_fwd / launches / (bwd_ms * 1e-3) / 1e12, 2)},
+        "kernels": kernels,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None},
         "device": {"name": prop.name, "cus": prop.multi_processor_count,

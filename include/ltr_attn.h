@@ -45,6 +45,8 @@ extern "C" {
 /* flags */
 #define LTR_CAUSAL 1u /* mask by global position */
 #define LTR_MERGE 2u  /* forward: o/lse hold an earlier partial result; merge into it */
+#define LTR_NO_DQ 4u    /* backward: skip the dQ kernel (dq may be NULL) */
+#define LTR_NO_DKDV 8u  /* backward: skip the dK/dV kernel (chunk[].dk/dv may be NULL) */
 
 /* error codes */
 #define LTR_OK 0
@@ -126,7 +128,10 @@ int ltr_attn_bwd_delta(const ltr_attn_delta_args *args, void *stream);
  * chunk[c].dv are fp32 ACCUMULATORS: the caller zero-fills them before the first
  * launch that contributes, launches on one stream accumulate (that is how dK/dV sum
  * over the Q chunks of several ranks), and ltr_cast_f32_to_bf16 makes the final cast.
- * dK/dV of a GQA group sum over its Hq/Hkv query heads.
+ * dK/dV of a GQA group sum over its Hq/Hkv query heads.  Two kernels are enqueued, one
+ * for dK/dV and one for dQ (no atomics: results are bitwise reproducible); LTR_NO_DQ /
+ * LTR_NO_DKDV enqueue only one of them, e.g. for a ring step where dK/dV travel with the
+ * KV chunk, or to time the kernels separately.
  */
 typedef struct ltr_attn_bwd_args {
     const void *q;
@@ -146,8 +151,8 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;
-    uint32_t flags;       /* LTR_CAUSAL */
-    int32_t io_dtype;     /* LTR_BF16 or LTR_F32 */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV */
+    int32_t io_dtype;     /* LTR_BF16 (the backward kernels are bf16 only) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
 } ltr_attn_bwd_args;

@@ -121,8 +121,9 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
-                        causal=False, scale=None):
-    """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs."""
+                        causal=False, scale=None, do_dq=True, do_dkdv=True):
+    """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
+    do_dq / do_dkdv select which of the two backward kernels are enqueued."""
     lib = _lib.load()
     _req(q, "q")
     _req(do, "dO")
@@ -142,7 +143,8 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     a.dk_stride, a.dv_stride = _s3(dk_accs[0]), _s3(dv_accs[0])
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
-    a.flags = _lib.LTR_CAUSAL if causal else 0
+    a.flags = ((_lib.LTR_CAUSAL if causal else 0) | (0 if do_dq else _lib.LTR_NO_DQ)
+               | (0 if do_dkdv else _lib.LTR_NO_DKDV))
     a.io_dtype = _DT[q.dtype]
     stream = _stream_ptr(q.device)
     n = len(ks)

@@ -1332,15 +1332,17 @@ extern "C" int ltr_attn_bwd_delta(const ltr_attn_delta_args *a, void *stream) {
 }
 
 extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
-    if (!a || !a->q || !a->d_o || !a->lse || !a->delta || !a->dq) return LTR_EINVAL;
+    if (!a || !a->q || !a->d_o || !a->lse || !a->delta) return LTR_EINVAL;
+    const bool do_dq = !(a->flags & LTR_NO_DQ), do_dkdv = !(a->flags & LTR_NO_DKDV);
+    if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~LTR_CAUSAL) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
     if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
-    if (!aligned16(a->q) || !aligned16(a->d_o) || !aligned16(a->dq)) return LTR_EALIGN;
+    if (!aligned16(a->q) || !aligned16(a->d_o) || (do_dq && !aligned16(a->dq))) return LTR_EALIGN;
     if (!strides_ok(a->q_stride, 2) || !strides_ok(a->do_stride, 2) || !strides_ok(a->k_stride, 2) ||
         !strides_ok(a->v_stride, 2) || !strides_ok(a->dk_stride, 4) || !strides_ok(a->dv_stride, 4))
         return LTR_EALIGN;
@@ -1350,9 +1352,10 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     long long tiles = 0;
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];
-        if (!ch.k || !ch.v || !ch.dk || !ch.dv || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk))
-            return LTR_EINVAL;
-        if (!aligned16(ch.k) || !aligned16(ch.v) || !aligned16(ch.dk) || !aligned16(ch.dv)) return LTR_EALIGN;
+        if (!ch.k || !ch.v || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
+        if (do_dkdv && (!ch.dk || !ch.dv)) return LTR_EINVAL;
+        if (!aligned16(ch.k) || !aligned16(ch.v)) return LTR_EALIGN;
+        if (do_dkdv && (!aligned16(ch.dk) || !aligned16(ch.dv))) return LTR_EALIGN;
         p.chunk[c].k = ch.k;
         p.chunk[c].v = ch.v;
         p.chunk[c].dk = (float *)ch.dk;
@@ -1398,11 +1401,11 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     const long long nblk_q = (long long)((p.Sq + 127) / 128) * p.B * p.Hq;
     if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
     if (a->D == 128) {
-        hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(256), BwdLds<128>::TOTAL, st, p);
-        hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
+        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(256), BwdLds<128>::TOTAL, st, p);
+        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
     } else {
-        hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(256), BwdLds<64>::TOTAL, st, p);
-        hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
+        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(256), BwdLds<64>::TOTAL, st, p);
+        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }

@@ -257,3 +257,58 @@ def n_pairs_causal(q_pos: torch.Tensor, k_pos: torch.Tensor) -> int:
     """Number of unmasked (query, key) pairs; positions sorted or not."""
     ks = torch.sort(k_pos).values
     return int(torch.searchsorted(ks, q_pos, right=True).sum())
+
+
+# --------------------------------------------------------------------------- sampled checks at full size
+def sampled_rows(q, k, v, q_pos, k_pos, causal, rows, do=None, dtype=torch.float64):
+    """Dense closed form restricted to sampled query rows, for inputs too large for the dense oracle.
+    q: [B,Sq,Hq,D]; k, v: [B,Sk,Hkv,D] (any row order; k_pos gives positions); rows: list of (b, h, i).
+    Returns per row (o [D], lse, dq [D] or None).  Pinned against dense_attention_grads in the CPU tests."""
+    D = q.shape[-1]
+    n_rep = q.shape[2] // k.shape[2]
+    scale = 1.0 / math.sqrt(D)
+    out = []
+    for (b, h, i) in rows:
+        g = h // n_rep
+        qi = q[b, i, h].to(dtype)
+        kk, vv = k[b, :, g].to(dtype), v[b, :, g].to(dtype)
+        s = (kk @ qi) * scale
+        if causal:
+            s = s.masked_fill(k_pos > q_pos[i], NEG_INF)
+        lse = torch.logsumexp(s, 0)
+        p = torch.exp(s - lse)
+        o = p @ vv
+        dq = None
+        if do is not None:
+            doi = do[b, i, h].to(dtype)
+            dp = vv @ doi
+            ds = p * (dp - (doi * o).sum())
+            dq = (ds @ kk) * scale
+        out.append((o, lse, dq))
+    return out
+
+
+def sampled_keys(q, k, v, o, lse, do, q_pos, k_pos, causal, keys, dtype=torch.float64):
+    """dK and dV of sampled keys (b, g, j) from the recompute formula over ALL query rows and the
+    n_rep query heads of the group, given the forward results o [B,Sq,Hq,D] and lse [B,Hq,Sq]."""
+    D = q.shape[-1]
+    n_rep = q.shape[2] // k.shape[2]
+    scale = 1.0 / math.sqrt(D)
+    out = []
+    for (b, g, j) in keys:
+        kj, vj = k[b, j, g].to(dtype), v[b, j, g].to(dtype)
+        dk = torch.zeros(D, dtype=dtype)
+        dv = torch.zeros(D, dtype=dtype)
+        for h in range(g * n_rep, (g + 1) * n_rep):
+            qq, dd, oo = q[b, :, h].to(dtype), do[b, :, h].to(dtype), o[b, :, h].to(dtype)
+            s = (qq @ kj) * scale
+            p = torch.exp(s - lse[b, h].to(dtype))
+            if causal:
+                p = torch.where(q_pos >= k_pos[j], p, torch.zeros_like(p))
+            p = torch.where(torch.isfinite(p), p, torch.zeros_like(p))
+            delta = (dd * oo).sum(-1)
+            ds = p * (dd @ vj - delta)
+            dk += (ds @ qq) * scale
+            dv += p @ dd
+        out.append((dk, dv))
+    return out

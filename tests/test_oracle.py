@@ -207,3 +207,19 @@ def test_fully_masked_rows_are_zero_and_minus_inf():
     assert torch.isinf(lse[0, 0, :2]).all() and (o[0, :2] == 0).all()
     d, dl = orc.dense_attention(q, k, v, torch.tensor([0, 1, 10, 11]), torch.tensor([5, 6, 7, 8]), True)
     assert (o[0, 2:] - d[0, 2:]).abs().max() < 1e-12
+
+
+def test_sampled_checks_match_dense():
+    q = _rand((2, 24, 4, 8), 40, torch.float64)
+    k, v = _rand((2, 24, 2, 8), 41, torch.float64), _rand((2, 24, 2, 8), 42, torch.float64)
+    do = _rand((2, 24, 4, 8), 43, torch.float64)
+    perm = torch.randperm(24, generator=torch.Generator().manual_seed(1))
+    qpos, kpos = torch.arange(24)[perm], torch.arange(24)
+    o, lse, dq, dk, dv = orc.dense_attention_grads(q[:, perm], k, v, do[:, perm], qpos, kpos, True)
+    rows = [(0, 0, 3), (1, 3, 23), (0, 2, 11)]
+    for (b, h, i), (ro, rl, rdq) in zip(rows, orc.sampled_rows(q[:, perm], k, v, qpos, kpos, True, rows, do[:, perm])):
+        assert (ro - o[b, i, h]).abs().max() < 1e-12 and abs(rl - lse[b, h, i]) < 1e-12
+        assert (rdq - dq[b, i, h]).abs().max() < 1e-12
+    keys = [(0, 0, 0), (1, 1, 17), (0, 1, 23)]
+    for (b, g, j), (rk, rv) in zip(keys, orc.sampled_keys(q[:, perm], k, v, o, lse, do[:, perm], qpos, kpos, True, keys)):
+        assert (rk - dk[b, j, g]).abs().max() < 1e-12 and (rv - dv[b, j, g]).abs().max() < 1e-12
