@@ -21,6 +21,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
+# HBM-side bytes per launch of bwd_dkdv_kernel<128> on config 3, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
+# command calibrated against streaming kernels of known size (profiles/bench_c3_counters.md)
+DKDV_C3_TRAFFIC_BYTES = 1.85e9
 
 
 def _workload(name):
@@ -237,7 +240,8 @@ def main():
         "frac_of_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         "kernels": kernels,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None},
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": DKDV_C3_TRAFFIC_BYTES if (args.workload == "c3" and bwd) else None},
         "device": {"name": prop.name, "cus": prop.multi_processor_count,
                    "clock_mhz": getattr(prop, "clock_rate", 0) // 1000},
     }
