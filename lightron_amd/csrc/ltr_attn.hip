@@ -147,6 +147,46 @@ __device__ __forceinline__ bf16x8 lds_operand_tr(const __bf16 *tile, int stride,
     return u.v;
 }
 
+// Block barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global
+// load (workgroup-scope fence), which would expose the latency of the tile prefetch that is meant to
+// stay in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Unpadded row-major LDS tile of D bf16 per row whose 16-byte chunks are XOR-swizzled: chunk c of row r
+// lives at chunk position c ^ lds_swz<D>(r).  LDS has 64 banks of 4 bytes; a 128-bit read is served 16
+// lanes at a time and a 64-bit (transpose) read 32 lanes at a time.  With this permutation both the MFMA
+// operand read (16 consecutive rows, same logical chunk) and the transpose read (4 consecutive rows x 4
+// consecutive chunks) touch every bank exactly once, and so does the staging store (one row per 16 lanes).
+template <int D>
+__device__ __forceinline__ int lds_swz(int row) {
+    return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+}
+
+template <int D>
+__device__ __forceinline__ int lds_swz_off(int row, int chunk) {   // element offset of (row, 16-byte chunk)
+    return row * D + ((chunk ^ lds_swz<D>(row)) << 3);
+}
+
+// transpose-read operand (same contract as lds_operand_tr) from a swizzled tile
+template <int D>
+__device__ __forceinline__ bf16x8 lds_operand_tr_swz(const __bf16 *tile, int k0, int n_base, int lane) {
+    const int li = lane & 15, g = lane >> 4;
+    const int hh = g >> 1;
+    const int col = n_base + ((g & 1) << 4) + ((li & 3) << 2);
+    const int row = k0 + 4 * hh + (li >> 2);
+    i16x4 lo = lds_read_tr16(tile + lds_swz_off<D>(row, col >> 3) + (col & 7));
+    i16x4 hi = lds_read_tr16(tile + lds_swz_off<D>(row + 8, col >> 3) + (col & 7));
+    union {
+        struct { i16x4 a, b; } s;
+        bf16x8 v;
+    } u;
+    u.s.a = lo;
+    u.s.b = hi;
+    return u.v;
+}
+
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) {
     union { uint4 u; bf16x8 v; } c;
     c.u = x;
@@ -590,214 +630,170 @@ __global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst
 
 // ------------------------------------------------------------------------------ backward, bf16
 // Two kernels, no atomics, bitwise reproducible:
-//   bwd_dkdv_kernel  a block owns 128 keys of one kv head (32 per wave; K and V operands live in
-//                    registers), loops over the query heads of the GQA group and over 64-row
-//                    query tiles staged in double-buffered LDS; dK^T and dV^T accumulate in
-//                    registers for the whole loop and are added to the fp32 accumulators once.
+//   bwd_dkdv_kernel  a block owns 128 keys of one kv head and runs 8 waves, two per SIMD: for each of
+//                    the four 32-key slices one "P wave" (S = Q K^T, P, dV^T += dO^T P; K operand in
+//                    registers) and one "dS wave" (dP = dO V^T, dS = P*(dP - DELTA), dK^T += Q^T dS;
+//                    V operand in registers).  The P wave hands P (bf16, accumulator layout) to its
+//                    partner through a 2 KB LDS slot; both GEMM pairs of a 32-row sub-tile are
+//                    separated by one block barrier.  The block loops over the query heads of the
+//                    GQA group and over 64-row Q / dO tiles staged in double-buffered LDS; dK^T and
+//                    dV^T stay in registers for the whole loop.
 //   bwd_dq_kernel    a block owns 128 query rows of one query head (32 per wave; Q and dO
 //                    operands in registers), loops over 64-key K/V tiles like the forward;
 //                    dQ^T accumulates in registers.
-// LDS of bwd_dkdv_kernel (dynamic): two buffers of {Q tile, dO tile, LSE*log2e, DELTA}.
+// LDS of bwd_dkdv_kernel (dynamic): two buffers of {Q tile, dO tile, LSE*log2e, DELTA}, then the P slots.
 template <int D>
 struct BwdLds {
-    static constexpr int BN = 128;      // keys per block, 32 per wave
-    static constexpr int BM = 64;       // query rows per iteration (two 32-row MFMA sub-tiles)
-    static constexpr int QS = D + 24;   // Q / dO tile row stride (elements): row + 48 B suits both the
-                                        // 128-bit operand reads and the transpose reads
-    static constexpr int TILE = BM * QS;                                 // elements
+    static constexpr int BN = 128;      // keys per block, 32 per wave pair
+    static constexpr int BM = 64;       // query rows per tile (two 32-row MFMA sub-tiles)
+    static constexpr int NT = 512;      // threads per block
+    static constexpr int TILE = BM * D;                                  // elements; rows unpadded, chunks swizzled
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, lse, delta
-    static constexpr int TOTAL = 2 * BUF_BYTES;
+    static constexpr int P_SLOT = 64 * 32;                               // one lane = 16 bf16 = 32 bytes
+    static constexpr int P_OFF = 2 * BUF_BYTES;
+    static constexpr int MAX_QTILES = 4096;                              // Sq <= 262144 per launch
+    static constexpr int LIST_OFF = P_OFF + 4 * 2 * P_SLOT;              // 4 slices x 2 parities of P slots
+    static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;     // two tile lists (ushort) + counts
 };
 
-// One 64-row iteration of bwd_dkdv_kernel for one wave (its 32 keys), as two 32-row sub-tiles a, b.
-// A sub-tile needs S = Q K^T and dP = dO V^T (query rows in accumulator registers, this lane's key in
-// the lane), then P = exp2(S*c2 - LSE*log2e) and dS = P*(dP - DELTA) element by element, then
-// dV^T += dO^T P and dK^T += Q^T dS with P / dS fed from registers as B operands and dO^T / Q^T read
-// from the same LDS tiles by transpose loads.  Order of issue:
-//     S_a, dP_a | S_b, dP_b + softmax(a) | dV, dK (a) + softmax(b) | dV, dK (b)
-// so the softmax arithmetic of one sub-tile sits between the MFMAs of another and the matrix pipe and
-// the VALU run concurrently inside a single wave; sched_barrier keeps the interleave.  MFMA results are
-// read once and P / dS go straight to packed bf16 pairs (never written back to the accumulator tile).
 struct BwdMaskCtx {
     bool key_ok, causal;
     int my_kpos, row_base, Sq, q_split, p0, p1;
 };
 
-// elements 2j and 2j+1 of a sub-tile: P and dS pairs
-template <bool MASK>
-__device__ __forceinline__ void bwd_softmax_pair(const f32x16 &s, const f32x16 &dp, int j, const f32x4 &lv, const f32x4 &dv,
-                                                 float c2, int r0, int hh, const BwdMaskCtx &m, PackedTile &pp,
-                                                 PackedTile &pds) {
-    float pv[2], dsv[2];
-#pragma unroll
-    for (int e = 0; e < 2; e++) {
-        const int r = 2 * j + e;
-        pv[e] = __builtin_amdgcn_exp2f(s[r] * c2 - lv[r % 4]);
-        dsv[e] = pv[e] * (dp[r] - dv[r % 4]);
-        if (MASK) {
-            const int qrow = m.row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
-            const int qpos = q_position(qrow, m.q_split, m.p0, m.p1);
-            const bool vis = m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
-            pv[e] = vis ? pv[e] : 0.f;
-            dsv[e] = vis ? dsv[e] : 0.f;
-        }
-    }
-    pp.u[j] = pack2_bf16(pv[0], pv[1]);
-    pds.u[j] = pack2_bf16(dsv[0], dsv[1]);
+__device__ __forceinline__ bool bwd_visible(const BwdMaskCtx &m, int r0, int r, int hh) {
+    const int qrow = m.row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
+    const int qpos = q_position(qrow, m.q_split, m.p0, m.p1);
+    return m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
 }
 
-template <int D, bool MASK>
-__device__ __forceinline__ void bwd_dkdv_tile(const __bf16 *Qs, const __bf16 *dOs, const float *lse_s, const float *dlt_s,
-                                              const bf16x8 (&kreg)[D / 16], const bf16x8 (&vreg)[D / 16],
-                                              f32x16 (&dkacc)[D / 32], f32x16 (&dvacc)[D / 32], const f32x16 &zero16,
-                                              int lane, int l32, int hh, float c2, const BwdMaskCtx &m) {
-    constexpr int QS = BwdLds<D>::QS;
-    constexpr int NK = D / 16, ND = D / 32;
-    f32x16 sa = zero16, dpa = zero16, sb = zero16, dpb = zero16;
-    PackedTile pa, dsa, pb, dsb;
-    const __bf16 *qrow = Qs + l32 * QS + 8 * hh;
-    const __bf16 *drow = dOs + l32 * QS + 8 * hh;
-    const float *lrow = lse_s + 4 * hh, *trow = dlt_s + 4 * hh;
+// P wave: S = Q K^T for rows r0..r0+31 of the tile
+template <int D>
+__device__ __forceinline__ void bwd_p_gemm_s(const __bf16 *Qs, const bf16x8 (&kreg)[D / 16], const f32x16 &zero16, int r0,
+                                             int l32, int hh, f32x16 &s) {
+    constexpr int NK = D / 16;
+    const __bf16 *qrow = Qs + (r0 + l32) * D;
+    const int sw = lds_swz<D>(r0 + l32) ^ hh;           // chunk 2*kb + hh lives at (2*kb) ^ sw
+    s = zero16;
+    bf16x8 qb[3];
+    qb[0] = *(const bf16x8 *)(qrow + ((0 ^ sw) << 3));
+    qb[1] = *(const bf16x8 *)(qrow + ((2 ^ sw) << 3));
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + 2 < NK) qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + (((2 * (kb + 2)) ^ sw) << 3));
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], s, 0, 0, 0);
+    }
+}
 
-    // S_a, dP_a (operands fetched two steps ahead of their MFMAs)
-    {
-        bf16x8 qb[3], db_[3];
-        qb[0] = *(const bf16x8 *)(qrow);
-        db_[0] = *(const bf16x8 *)(drow);
-        qb[1] = *(const bf16x8 *)(qrow + 16);
-        db_[1] = *(const bf16x8 *)(drow + 16);
+// P wave: P = exp2(S*c2 - LSE*log2e) -> packed bf16 in accumulator layout
+template <bool MASK>
+__device__ __forceinline__ void bwd_p_softmax(const f32x16 &s, const float *lse_s, int r0, int hh, float c2,
+                                              const BwdMaskCtx &m, PackedTile &pp) {
 #pragma unroll
-        for (int kb = 0; kb < NK; kb++) {
-            if (kb + 2 < NK) {
-                qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + (kb + 2) * 16);
-                db_[(kb + 2) % 3] = *(const bf16x8 *)(drow + (kb + 2) * 16);
-            }
-            sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], sa, 0, 0, 0);
-            dpa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db_[kb % 3], vreg[kb], dpa, 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+    for (int g = 0; g < 4; g++) {
+        const f32x4 lv = *(const f32x4 *)(lse_s + r0 + 8 * g + 4 * hh);
+        float pv[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            pv[e] = __builtin_amdgcn_exp2f(s[4 * g + e] * c2 - lv[e]);
+            if (MASK) pv[e] = bwd_visible(m, r0, 4 * g + e, hh) ? pv[e] : 0.f;
+        }
+        pp.u[2 * g] = pack2_bf16(pv[0], pv[1]);
+        pp.u[2 * g + 1] = pack2_bf16(pv[2], pv[3]);
+    }
+}
+
+// P wave, second half: dV^T += dO^T P
+template <int D>
+__device__ __forceinline__ void bwd_p_phase2(const __bf16 *dOs, f32x16 (&dvacc)[D / 32], int r0, int lane,
+                                             const PackedTile &pp) {
+    constexpr int ND = D / 32;
+    bf16x8 ao = lds_operand_tr_swz<D>(dOs, r0, 0, lane);
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+        const bf16x8 pop = operand_of(pp, kb);
+#pragma unroll
+        for (int db = 0; db < ND; db++) {
+            const int step = kb * ND + db;
+            bf16x8 aon = ao;
+            if (step + 1 < 2 * ND) aon = lds_operand_tr_swz<D>(dOs, r0 + ((step + 1) / ND) * 16, ((step + 1) % ND) * 32, lane);
+            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pop, dvacc[db], 0, 0, 0);
+            ao = aon;
         }
     }
-    // S_b, dP_b with softmax(a): 8 pairs over 2*NK MFMAs
-    {
-        f32x4 lv = *(const f32x4 *)(lrow), dv = *(const f32x4 *)(trow);
-        bf16x8 qb[3], db_[3];
-        qb[0] = *(const bf16x8 *)(qrow + 32 * QS);
-        db_[0] = *(const bf16x8 *)(drow + 32 * QS);
-        qb[1] = *(const bf16x8 *)(qrow + 32 * QS + 16);
-        db_[1] = *(const bf16x8 *)(drow + 32 * QS + 16);
+}
+
+// dS wave, first half: dP = dO V^T
+template <int D>
+__device__ __forceinline__ void bwd_ds_phase1(const __bf16 *dOs, const bf16x8 (&vreg)[D / 16], const f32x16 &zero16, int r0,
+                                              int l32, int hh, f32x16 &dp) {
+    constexpr int NK = D / 16;
+    const __bf16 *drow = dOs + (r0 + l32) * D;
+    const int sw = lds_swz<D>(r0 + l32) ^ hh;
+    dp = zero16;
+    bf16x8 db_[3];
+    db_[0] = *(const bf16x8 *)(drow + ((0 ^ sw) << 3));
+    db_[1] = *(const bf16x8 *)(drow + ((2 ^ sw) << 3));
 #pragma unroll
-        for (int kb = 0; kb < NK; kb++) {
-            constexpr int PPS = 8 / NK > 0 ? 8 / NK : 1;    // pairs per kb step (1 for D=128, 2 for D=64)
-            if (kb + 2 < NK) {
-                qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + 32 * QS + (kb + 2) * 16);
-                db_[(kb + 2) % 3] = *(const bf16x8 *)(drow + 32 * QS + (kb + 2) * 16);
-            }
-            f32x4 lvn = lv, dvn = dv;
-            {
-                const int jn = (kb + 1) * PPS;              // first pair of the next step
-                if (jn < 8 && jn % 2 == 0) {
-                    lvn = *(const f32x4 *)(lrow + 8 * (jn / 2));
-                    dvn = *(const f32x4 *)(trow + 8 * (jn / 2));
-                }
-            }
-            sb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], sb, 0, 0, 0);
-#pragma unroll
-            for (int q = 0; q < PPS; q++) {
-                const int j = kb * PPS + q;
-                if (j < 8) {
-                    if (q > 0 && j % 2 == 0) {              // D = 64: a new row group inside the step
-                        lv = *(const f32x4 *)(lrow + 8 * (j / 2));
-                        dv = *(const f32x4 *)(trow + 8 * (j / 2));
-                    }
-                    bwd_softmax_pair<MASK>(sa, dpa, j, lv, dv, c2, 0, hh, m, pa, dsa);
-                }
-            }
-            dpb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db_[kb % 3], vreg[kb], dpb, 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            lv = lvn;
-            dv = dvn;
-        }
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + 2 < NK) db_[(kb + 2) % 3] = *(const bf16x8 *)(drow + (((2 * (kb + 2)) ^ sw) << 3));
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db_[kb % 3], vreg[kb], dp, 0, 0, 0);
     }
-    // dV, dK of sub-tile a with softmax(b): 8 pairs over 2*ND steps of two MFMAs
-    {
-        f32x4 lv = *(const f32x4 *)(lrow + 32), dv = *(const f32x4 *)(trow + 32);
-        bf16x8 ao = lds_operand_tr(dOs, QS, 0, 0, lane), aq = lds_operand_tr(Qs, QS, 0, 0, lane);
+}
+
+// dS wave: dS = P * (dP - DELTA) with P from the partner's LDS slot -> packed bf16
+__device__ __forceinline__ void bwd_ds_softmax(const float *dlt_s, const unsigned *pslot, const f32x16 &dp, int r0, int lane,
+                                               int hh, PackedTile &ds) {
+    const uint4 p0 = *(const uint4 *)(pslot + lane * 8), p1 = *(const uint4 *)(pslot + lane * 8 + 4);
+    const unsigned pu[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            const bf16x8 pop = operand_of(pa, kb), dsop = operand_of(dsa, kb);
+    for (int g = 0; g < 4; g++) {
+        const f32x4 dv = *(const f32x4 *)(dlt_s + r0 + 8 * g + 4 * hh);
+        float dsv[4];
 #pragma unroll
-            for (int db = 0; db < ND; db++) {
-                const int step = kb * ND + db;
-                constexpr int PPS = 8 / (2 * ND);           // pairs per step (1 for D=128, 2 for D=64)
-                bf16x8 aon = ao, aqn = aq;
-                if (step + 1 < 2 * ND) {
-                    const int nkb = (step + 1) / ND, ndb = (step + 1) % ND;
-                    aon = lds_operand_tr(dOs, QS, nkb * 16, ndb * 32, lane);
-                    aqn = lds_operand_tr(Qs, QS, nkb * 16, ndb * 32, lane);
-                } else {                                    // first operands of the sub-tile b phase
-                    aon = lds_operand_tr(dOs, QS, 32, 0, lane);
-                    aqn = lds_operand_tr(Qs, QS, 32, 0, lane);
-                }
-                f32x4 lvn = lv, dvn = dv;
-                {
-                    const int jn = (step + 1) * PPS;
-                    if (jn < 8 && jn % 2 == 0) {
-                        lvn = *(const f32x4 *)(lrow + 32 + 8 * (jn / 2));
-                        dvn = *(const f32x4 *)(trow + 32 + 8 * (jn / 2));
-                    }
-                }
-                dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pop, dvacc[db], 0, 0, 0);
-#pragma unroll
-                for (int q = 0; q < PPS; q++) {
-                    const int j = step * PPS + q;
-                    if (q > 0 && j % 2 == 0) {
-                        lv = *(const f32x4 *)(lrow + 32 + 8 * (j / 2));
-                        dv = *(const f32x4 *)(trow + 32 + 8 * (j / 2));
-                    }
-                    bwd_softmax_pair<MASK>(sb, dpb, j, lv, dv, c2, 32, hh, m, pb, dsb);
-                }
-                dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsop, dkacc[db], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                ao = aon;
-                aq = aqn;
-                lv = lvn;
-                dv = dvn;
-            }
+        for (int e = 0; e < 4; e++) {
+            const unsigned u = pu[2 * g + e / 2];
+            const float pv = __uint_as_float((e & 1) ? (u & 0xffff0000u) : (u << 16));   // masked entries are 0
+            dsv[e] = pv * (dp[4 * g + e] - dv[e]);
         }
-        // dV, dK of sub-tile b
+        ds.u[2 * g] = pack2_bf16(dsv[0], dsv[1]);
+        ds.u[2 * g + 1] = pack2_bf16(dsv[2], dsv[3]);
+    }
+}
+
+// dS wave: dK^T += Q^T dS
+template <int D>
+__device__ __forceinline__ void bwd_ds_gemm_dk(const __bf16 *Qs, f32x16 (&dkacc)[D / 32], int r0, int lane,
+                                               const PackedTile &ds) {
+    constexpr int ND = D / 32;
+    bf16x8 aq = lds_operand_tr_swz<D>(Qs, r0, 0, lane);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            const bf16x8 pop = operand_of(pb, kb), dsop = operand_of(dsb, kb);
+    for (int kb = 0; kb < 2; kb++) {
+        const bf16x8 dsop = operand_of(ds, kb);
 #pragma unroll
-            for (int db = 0; db < ND; db++) {
-                const int step = kb * ND + db;
-                bf16x8 aon = ao, aqn = aq;
-                if (step + 1 < 2 * ND) {
-                    const int nkb = (step + 1) / ND, ndb = (step + 1) % ND;
-                    aon = lds_operand_tr(dOs, QS, 32 + nkb * 16, ndb * 32, lane);
-                    aqn = lds_operand_tr(Qs, QS, 32 + nkb * 16, ndb * 32, lane);
-                }
-                dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pop, dvacc[db], 0, 0, 0);
-                dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsop, dkacc[db], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                ao = aon;
-                aq = aqn;
-            }
+        for (int db = 0; db < ND; db++) {
+            const int step = kb * ND + db;
+            bf16x8 aqn = aq;
+            if (step + 1 < 2 * ND) aqn = lds_operand_tr_swz<D>(Qs, r0 + ((step + 1) / ND) * 16, ((step + 1) % ND) * 32, lane);
+            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsop, dkacc[db], 0, 0, 0);
+            aq = aqn;
         }
     }
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
+__global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     using L = BwdLds<D>;
-    constexpr int BN = L::BN, BM = L::BM, QS = L::QS;
+    constexpr int BN = L::BN, BM = L::BM, NT = L::NT;
     constexpr int CPR = D / 8;
-    constexpr int NLD = BM * CPR / 256;  // 16-byte chunks per thread per tile (4 for D=128, 2 for D=64)
-    constexpr int RPL = 256 / CPR;       // rows covered by one pass of the block's 256 threads
+    constexpr int NLD = BM * CPR / NT;   // 16-byte chunks per thread per tile and tensor (2 for D=128, 1 for D=64)
+    constexpr int RPL = NT / CPR;        // rows covered by one pass of the block's threads
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slice = w & 3;             // 32-key slice; waves w and w+4 (same SIMD) are partners
+    const bool p_role = w < 4;           // P wave (S, P, dV) or dS wave (dP, dS, dK)
     const int l32 = lane & 31, hh = lane >> 5;
     const bool causal = p.flags & LTR_CAUSAL;
 
@@ -822,46 +818,38 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     if (c >= p.n_chunks) return;
     const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
     const int key0 = kt * BN;
-    const int my_key = key0 + w * 32 + l32;     // this lane's key in S / dP / dK^T / dV^T tiles
+    const int my_key = key0 + slice * 32 + l32;   // this lane's key in S / dP / dK^T / dV^T tiles
     const bool key_ok = my_key < sk;
-    const int my_kpos = pos0 + my_key;
     const int tile_kpos_lo = pos0 + key0;
     const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
     const bool key_tail = key0 + BN > sk;
 
-    // resident B operands of S = Q K^T and dP = dO V^T: lane (key l32, half hh) holds d = 16*kb + 8*hh .. +7
-    bf16x8 kreg[D / 16], vreg[D / 16];
+    // resident B operand: K rows for a P wave, V rows for a dS wave; lane (key l32, half hh) holds
+    // d = 16*kb + 8*hh .. +7
+    bf16x8 kvreg[D / 16];
     {
-        const __bf16 *kp = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
-        const __bf16 *vp = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+        const __bf16 *base = p_role ? (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2]
+                                    : (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+        const long long rs = p_role ? p.ks[1] : p.vs[1];
         const int ksafe = min(my_key, sk - 1);
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
-            uint4 kx = *(const uint4 *)(kp + (long long)ksafe * p.ks[1] + kb * 16 + 8 * hh);
-            uint4 vx = *(const uint4 *)(vp + (long long)ksafe * p.vs[1] + kb * 16 + 8 * hh);
-            if (!key_ok) {
-                kx = make_uint4(0, 0, 0, 0);
-                vx = make_uint4(0, 0, 0, 0);
-            }
-            kreg[kb] = as_bf16x8(kx);
-            vreg[kb] = as_bf16x8(vx);
+            uint4 x = *(const uint4 *)(base + (long long)ksafe * rs + kb * 16 + 8 * hh);
+            if (!key_ok) x = make_uint4(0, 0, 0, 0);
+            kvreg[kb] = as_bf16x8(x);
         }
     }
 
     f32x16 zero16;
 #pragma unroll
     for (int r = 0; r < 16; r++) zero16[r] = 0.f;
-    f32x16 dkacc[D / 32], dvacc[D / 32];
+    f32x16 acc[D / 32];                  // dV^T (P wave) or dK^T (dS wave)
 #pragma unroll
-    for (int i = 0; i < D / 32; i++) {
-        dkacc[i] = zero16;
-        dvacc[i] = zero16;
-    }
+    for (int i = 0; i < D / 32; i++) acc[i] = zero16;
     const float c2 = p.scale * LTR_LOG2E;
 
-    // iteration space: (query head of the group, 64-row query tile).  A tile's class depends on its
-    // rows only: 0 = no row sees any key of the block (skipped); 1 = every (row, key) pair is visible;
-    // 2 = needs the mask (diagonal, tails).
+    // A tile's class depends on its rows only: 0 = no row sees any key of the block (skipped);
+    // 1 = every (row, key) pair is visible; 2 = needs the mask (diagonal, tails).
     auto tile_class = [&](int qt) {
         const int row0 = qt * BM;
         const bool edge = key_tail || row0 + BM > p.Sq;
@@ -872,6 +860,29 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         return (edge || tile_kpos_hi > lo) ? 2 : 1;
     };
 
+    // The q tiles of each class are listed once per block (wave 0, ballot compaction: the order, and with it
+    // the rounding of the accumulation, is fixed), so the main loops carry no classification arithmetic.
+    unsigned short *const tlist = (unsigned short *)(smem + L::LIST_OFF);     // [2][MAX_QTILES]
+    int *const tcount = (int *)(smem + L::LIST_OFF + 2 * L::MAX_QTILES * 2);
+    if (w == 0) {
+        int n1 = 0, n2 = 0;
+        for (int base = 0; base < p.n_qtiles; base += 64) {
+            const int qt = base + lane;
+            const int cls = qt < p.n_qtiles ? tile_class(qt) : 0;
+            const unsigned long long m1 = __builtin_amdgcn_ballot_w64(cls == 1), m2 = __builtin_amdgcn_ballot_w64(cls == 2);
+            const unsigned long long below = (1ull << lane) - 1ull;
+            if (cls == 1) tlist[n1 + __builtin_popcountll(m1 & below)] = (unsigned short)qt;
+            if (cls == 2) tlist[L::MAX_QTILES + n2 + __builtin_popcountll(m2 & below)] = (unsigned short)qt;
+            n1 += __builtin_popcountll(m1);
+            n2 += __builtin_popcountll(m2);
+        }
+        if (lane == 0) {
+            tcount[0] = n1;
+            tcount[1] = n2;
+        }
+    }
+    __syncthreads();
+
     // per-thread staging coordinates: row (tid / CPR) + RPL*i, 16-byte chunk tid % CPR
     const int ld_r = tid / CPR, ld_c = tid % CPR;
     const unsigned q_voff = (unsigned)(ld_r * (int)p.qs[1] + ld_c * 8);
@@ -880,26 +891,29 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     uint4 qld[NLD], dld[NLD];
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
+    unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 2 * (L::P_SLOT / 4);
 
     // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
     // live in straight-line loop bodies and the unmasked pass carries no bounds checks at all
     auto run_pass = [&](auto mask_tag) {
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr int cls = MASK ? 2 : 1;
+        const int cnt = __builtin_amdgcn_readfirstlane(tcount[cls - 1]);
+        const unsigned short *const list = tlist + (cls - 1) * L::MAX_QTILES;
+        int li_ = -1;                                 // index into the list
         auto advance = [&](int &rep, int &qt) {   // next tile of this class after (rep, qt); false when done
-            for (;;) {
-                if (++qt >= p.n_qtiles) {
-                    qt = 0;
-                    if (++rep >= p.n_rep) return false;
-                }
-                if (tile_class(qt) == cls) return true;
+            if (++li_ >= cnt) {
+                li_ = 0;
+                if (++rep >= p.n_rep) return false;
             }
+            qt = __builtin_amdgcn_readfirstlane((int)list[li_]);
+            return true;
         };
         auto gload = [&](int rep, int qt) {
             const int h = hkv * p.n_rep + rep;
             const int row0 = qt * BM;
-            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2] + (long long)row0 * p.qs[1];
-            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2] + (long long)row0 * p.dos[1];
+            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2] + (long long)(row0 * (int)p.qs[1]);
+            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2] + (long long)(row0 * (int)p.dos[1]);
             const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
             const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
             if (!MASK) {
@@ -935,8 +949,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             float *st = (float *)(dOs + L::TILE);
 #pragma unroll
             for (int i = 0; i < NLD; i++) {
-                *(uint4 *)(Qs + (ld_r + i * RPL) * QS + ld_c * 8) = qld[i];
-                *(uint4 *)(dOs + (ld_r + i * RPL) * QS + ld_c * 8) = dld[i];
+                *(uint4 *)(Qs + lds_swz_off<D>(ld_r + i * RPL, ld_c)) = qld[i];
+                *(uint4 *)(dOs + lds_swz_off<D>(ld_r + i * RPL, ld_c)) = dld[i];
             }
             if (tid < 2 * BM) {
                 float x = sld * st_mul;
@@ -949,52 +963,104 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         BwdMaskCtx mctx;
         mctx.key_ok = key_ok;
         mctx.causal = causal;
-        mctx.my_kpos = my_kpos;
+        mctx.my_kpos = pos0 + my_key;
         mctx.Sq = p.Sq;
         mctx.q_split = p.q_split;
         mctx.p0 = p.q_pos0[0];
         mctx.p1 = p.q_pos0[1];
-        int rep = 0, qt = -1;
-        if (!advance(rep, qt)) return;
+        if (cnt == 0) return;
+        int rep = 0, qt = 0;
+        advance(rep, qt);
         __syncthreads();   // the previous pass has finished reading LDS
         gload(rep, qt);
         lds_store(0);
         __syncthreads();
+        // Steps are numbered over the stream of 32-row sub-tiles, one LDS barrier per step.  In step k the P
+        // wave does all its work on sub-tile k (S, P -> slot k & 1, dV) and the dS wave all its work on
+        // sub-tile k-1 (dP, dS with P from the slot filled one step earlier, dK): inside a step the two waves
+        // of a SIMD are independent, so one wave's softmax arithmetic runs under the other's MFMAs.  Slot
+        // (k & 1) is rewritten in step k+2, after the barrier that ends step k+1 in which it was read.  Tile
+        // t+1 is fetched into registers in step 2t and stored to the LDS buffer of tile t-1 in step 2t+1,
+        // after the barrier that ends step 2t, the last one that reads tile t-1.  Both roles execute
+        // 2T + 1 barriers.
+        unsigned *const slot0 = pslot_base, *const slot1 = pslot_base + L::P_SLOT / 4;
+        auto put_slot = [&](unsigned *slot, const PackedTile &t) {
+            *(uint4 *)(slot + lane * 8) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
+            *(uint4 *)(slot + lane * 8 + 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
+        };
         int par = 0;
-        for (bool more = true; more;) {
-            mctx.row_base = qt * BM;
-            more = advance(rep, qt);
+        if (p_role) {
+            for (bool more = true; more;) {
+                mctx.row_base = qt * BM;
+                more = advance(rep, qt);
+                if (more) gload(rep, qt);
+                const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
+                const __bf16 *dOs = Qs + L::TILE;
+                const float *lse_s = (const float *)(dOs + L::TILE);
+                f32x16 s;
+                PackedTile pp;
+                bwd_p_gemm_s<D>(Qs, kvreg, zero16, 0, l32, hh, s);
+                bwd_p_softmax<MASK>(s, lse_s, 0, hh, c2, mctx, pp);
+                put_slot(slot0, pp);
+                bwd_p_phase2<D>(dOs, acc, 0, lane, pp);
+                lds_barrier();
+                bwd_p_gemm_s<D>(Qs, kvreg, zero16, 32, l32, hh, s);
+                bwd_p_softmax<MASK>(s, lse_s, 32, hh, c2, mctx, pp);
+                put_slot(slot1, pp);
+                bwd_p_phase2<D>(dOs, acc, 32, lane, pp);
+                if (more) lds_store(par ^ 1);
+                lds_barrier();
+                par ^= 1;
+            }
+            lds_barrier();                         // step 2T: only the dS waves have work
+        } else {
+            bool more = advance(rep, qt);          // step 0: staging duties only
             if (more) gload(rep, qt);
-            const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
-            const __bf16 *dOs = Qs + L::TILE;
-            const float *lse_s = (const float *)(dOs + L::TILE);
-            const float *dlt_s = lse_s + BM;
-            bwd_dkdv_tile<D, MASK>(Qs, dOs, lse_s, dlt_s, kreg, vreg, dkacc, dvacc, zero16, lane, l32, hh, c2, mctx);
-            if (more) lds_store(par ^ 1);
-            __syncthreads();
-            par ^= 1;
+            lds_barrier();
+            for (;;) {
+                const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
+                const __bf16 *dOs = Qs + L::TILE;
+                const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
+                f32x16 dp;
+                PackedTile ds;
+                // step 2t+1: sub-tile 0 of tile t
+                bwd_ds_phase1<D>(dOs, kvreg, zero16, 0, l32, hh, dp);
+                bwd_ds_softmax(dlt_s, slot0, dp, 0, lane, hh, ds);
+                bwd_ds_gemm_dk<D>(Qs, acc, 0, lane, ds);
+                if (more) lds_store(par ^ 1);
+                lds_barrier();
+                // step 2t+2: sub-tile 1 of tile t; fetch tile t+2
+                const bool had_next = more;
+                if (more) {
+                    more = advance(rep, qt);
+                    if (more) gload(rep, qt);
+                }
+                bwd_ds_phase1<D>(dOs, kvreg, zero16, 32, l32, hh, dp);
+                bwd_ds_softmax(dlt_s, slot1, dp, 32, lane, hh, ds);
+                bwd_ds_gemm_dk<D>(Qs, acc, 32, lane, ds);
+                lds_barrier();
+                par ^= 1;
+                if (!had_next) break;
+            }
         }
     };
     run_pass(std::false_type{});
     run_pass(std::true_type{});
 
-    // dK^T / dV^T tiles: lane (key l32 of this wave, half hh), register r -> d = 32*db + 8*(r/4) + 4hh + r%4
+    // dV^T (P wave) / dK^T (dS wave) tile: lane (key l32 of the slice, half hh), register r -> d = 32*db + 8*(r/4) + 4hh + r%4
     if (key_ok) {
-        float *dkp = p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2];
-        float *dvp = p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2];
+        float *gp = p_role ? p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2]
+                           : p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2];
+        const float mul = p_role ? 1.f : p.scale;
 #pragma unroll
         for (int db = 0; db < D / 32; db++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int d = db * 32 + 8 * g + 4 * hh;
-                f32x4 ok = *(const f32x4 *)(dkp + d), ov = *(const f32x4 *)(dvp + d);
+                f32x4 old = *(const f32x4 *)(gp + d);
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    ok[e] += dkacc[db][4 * g + e] * p.scale;
-                    ov[e] += dvacc[db][4 * g + e];
-                }
-                *(f32x4 *)(dkp + d) = ok;
-                *(f32x4 *)(dvp + d) = ov;
+                for (int e = 0; e < 4; e++) old[e] += acc[db][4 * g + e] * mul;
+                *(f32x4 *)(gp + d) = old;
             }
     }
 }
@@ -1362,6 +1428,8 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
         return LTR_EALIGN;
     for (int i = 0; i < 3; i++)
         if (a->dq_stride[i] < 0) return LTR_EINVAL;
+    if ((a->Sq + 63) / 64 > BwdLds<128>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
+    if ((a->Sq + 64) * a->q_stride[1] >= 0x7fffffffLL || (a->Sq + 64) * a->do_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     BwdParams p;
     long long tiles = 0;
     for (int c = 0; c < a->n_chunks; c++) {
@@ -1415,10 +1483,10 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     const long long nblk_q = (long long)((p.Sq + 127) / 128) * p.B * p.Hq;
     if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
     if (a->D == 128) {
-        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(256), BwdLds<128>::TOTAL, st, p);
+        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
         if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
     } else {
-        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(256), BwdLds<64>::TOTAL, st, p);
+        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
         if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
