@@ -293,30 +293,39 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     constexpr float LAZY = 8.f;
 
     // tile iterator over (chunk, key tile)
-    int c = 0, t = 0, nt = 0;
-    auto ntiles_of = [&](int ci) {
-        int sk = p.chunk[ci].sk;
-        int nvis = causal ? max(0, min(sk, blk_hi - p.chunk[ci].pos0 + 1)) : sk;
-        return (nvis + BN - 1) / BN;
-    };
+    // The fields of the chunk being loaded live in scalar registers and are re-read from the argument
+    // table only when the chunk changes (a scalar load per tile would share the LDS wait counter).
+    int c = -1, t = 0, nt = 0;
+    int ld_sk = 0, ld_pos0 = 0;
+    const __bf16 *ld_kb = nullptr, *ld_vb = nullptr;
     auto settle = [&]() {
         while (c < p.n_chunks && t >= nt) {
             c++;
             t = 0;
-            if (c < p.n_chunks) nt = ntiles_of(c);
+            if (c < p.n_chunks) {
+                ld_sk = p.chunk[c].sk;
+                ld_pos0 = p.chunk[c].pos0;
+                ld_kb = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+                ld_vb = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+                const int nvis = causal ? max(0, min(ld_sk, blk_hi - ld_pos0 + 1)) : ld_sk;
+                nt = (nvis + BN - 1) / BN;
+            }
         }
     };
-    nt = ntiles_of(0);
     settle();
 
     const int ld_r = tid / CPR, ld_c = tid % CPR;
     constexpr int RPL = 256 / CPR;
     const unsigned kvo = (unsigned)(ld_r * (int)p.ks[1] + ld_c * 8), vvo = (unsigned)(ld_r * (int)p.vs[1] + ld_c * 8);
     uint4 kld[NLD], vld[NLD];
-    auto gload = [&](int ci, int ti) {
-        const int sk = p.chunk[ci].sk;
-        const __bf16 *kp = (const __bf16 *)p.chunk[ci].k + b * p.ks[0] + hkv * p.ks[2] + (long long)(ti * BN) * p.ks[1];
-        const __bf16 *vp = (const __bf16 *)p.chunk[ci].v + b * p.vs[0] + hkv * p.vs[2] + (long long)(ti * BN) * p.vs[1];
+    int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
+    auto gload = [&](int ti) {
+        const int sk = ld_sk;
+        nx_sk = ld_sk;
+        nx_pos0 = ld_pos0;
+        nx_key0 = ti * BN;
+        const __bf16 *kp = ld_kb + (long long)(ti * BN * (int)p.ks[1]);
+        const __bf16 *vp = ld_vb + (long long)(ti * BN * (int)p.vs[1]);
         if (ti * BN + BN <= sk) {
 #pragma unroll
             for (int i = 0; i < NLD; i++) {
@@ -338,9 +347,9 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     };
 
     bool have = c < p.n_chunks;
-    if (have) gload(c, t);
+    if (have) gload(t);
     while (have) {
-        const int cc = c, ct = t;
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
@@ -351,10 +360,8 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
-        if (have_next) gload(c, t);
+        if (have_next) gload(t);
 
-        const int sk = p.chunk[cc].sk, pos0 = p.chunk[cc].pos0;
-        const int key0 = ct * BN;
         f32x16 s[2];
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
@@ -1134,29 +1141,38 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     for (int i = 0; i < D / 32; i++) dqacc[i] = zero16;
     const float c2 = p.scale * LTR_LOG2E;
 
-    int c = 0, t = 0, nt = 0;
-    auto ntiles_of = [&](int ci) {
-        int sk = p.chunk[ci].sk;
-        int nvis = causal ? max(0, min(sk, blk_hi - p.chunk[ci].pos0 + 1)) : sk;
-        return (nvis + BN - 1) / BN;
-    };
+    // The fields of the chunk being loaded live in scalar registers and are re-read from the argument
+    // table only when the chunk changes (a scalar load per tile would share the LDS wait counter).
+    int c = -1, t = 0, nt = 0;
+    int ld_sk = 0, ld_pos0 = 0;
+    const __bf16 *ld_kb = nullptr, *ld_vb = nullptr;
     auto settle = [&]() {
         while (c < p.n_chunks && t >= nt) {
             c++;
             t = 0;
-            if (c < p.n_chunks) nt = ntiles_of(c);
+            if (c < p.n_chunks) {
+                ld_sk = p.chunk[c].sk;
+                ld_pos0 = p.chunk[c].pos0;
+                ld_kb = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+                ld_vb = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+                const int nvis = causal ? max(0, min(ld_sk, blk_hi - ld_pos0 + 1)) : ld_sk;
+                nt = (nvis + BN - 1) / BN;
+            }
         }
     };
-    nt = ntiles_of(0);
     settle();
 
     const int ld_r = tid / CPR, ld_c = tid % CPR;
     constexpr int RPL = 256 / CPR;
     uint4 kld[NLD], vld[NLD];
-    auto gload = [&](int ci, int ti) {
-        const int sk = p.chunk[ci].sk;
-        const __bf16 *kp = (const __bf16 *)p.chunk[ci].k + b * p.ks[0] + hkv * p.ks[2] + (long long)(ti * BN) * p.ks[1];
-        const __bf16 *vp = (const __bf16 *)p.chunk[ci].v + b * p.vs[0] + hkv * p.vs[2] + (long long)(ti * BN) * p.vs[1];
+    int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
+    auto gload = [&](int ti) {
+        const int sk = ld_sk;
+        nx_sk = ld_sk;
+        nx_pos0 = ld_pos0;
+        nx_key0 = ti * BN;
+        const __bf16 *kp = ld_kb + (long long)(ti * BN * (int)p.ks[1]);
+        const __bf16 *vp = ld_vb + (long long)(ti * BN * (int)p.vs[1]);
         const unsigned kvo = (unsigned)(ld_r * (int)p.ks[1] + ld_c * 8), vvo = (unsigned)(ld_r * (int)p.vs[1] + ld_c * 8);
         if (ti * BN + BN <= sk) {
 #pragma unroll
@@ -1178,9 +1194,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     };
 
     bool have = c < p.n_chunks;
-    if (have) gload(c, t);
+    if (have) gload(t);
     while (have) {
-        const int cc = c, ct = t;
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
@@ -1191,10 +1207,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
-        if (have_next) gload(c, t);
+        if (have_next) gload(t);
 
-        const int sk = p.chunk[cc].sk, pos0 = p.chunk[cc].pos0;
-        const int key0 = ct * BN;
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         // two 32-key halves one after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
         // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic
@@ -1333,6 +1347,8 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
         const ltr_kv_chunk &ch = a->chunk[c];
         if (!ch.k || !ch.v || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
         if (!aligned16(ch.k) || !aligned16(ch.v)) return LTR_EALIGN;
+        // tile offsets inside a chunk are 32-bit element counts
+        if ((ch.sk + 64) * a->k_stride[1] >= 0x7fffffffLL || (ch.sk + 64) * a->v_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
         p.chunk[c].k = ch.k;
         p.chunk[c].v = ch.v;
         p.chunk[c].dk = nullptr;
@@ -1436,6 +1452,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
         const ltr_kv_chunk &ch = a->chunk[c];
         if (!ch.k || !ch.v || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
         if (do_dkdv && (!ch.dk || !ch.dv)) return LTR_EINVAL;
+        if ((ch.sk + 64) * a->k_stride[1] >= 0x7fffffffLL || (ch.sk + 64) * a->v_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
         if (!aligned16(ch.k) || !aligned16(ch.v)) return LTR_EALIGN;
         if (do_dkdv && (!aligned16(ch.dk) || !aligned16(ch.dv))) return LTR_EALIGN;
         p.chunk[c].k = ch.k;
