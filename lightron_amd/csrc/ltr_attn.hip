@@ -362,15 +362,17 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         const bool have_next = c < p.n_chunks;
         if (have_next) gload(t);
 
+        // the two key blocks accumulate in alternation: a dependent MFMA cannot issue until its predecessor
+        // has left the pipe, so every chain needs an independent one to fill the gap
         f32x16 s[2];
+        s[0] = zero16;
+        s[1] = zero16;
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-            s[nb] = zero16;
-#pragma unroll
-            for (int kb = 0; kb < D / 16; kb++) {
-                bf16x8 a = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
-                s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
-            }
+        for (int kb = 0; kb < D / 16; kb++) {
+            const bf16x8 a0 = *(const bf16x8 *)(Ks + l32 * KS + kb * 16 + 8 * hh);
+            const bf16x8 a1 = *(const bf16x8 *)(Ks + (32 + l32) * KS + kb * 16 + 8 * hh);
+            s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qreg[kb], s[0], 0, 0, 0);
+            s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qreg[kb], s[1], 0, 0, 0);
         }
         // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
@@ -657,9 +659,10 @@ struct BwdLds {
     static constexpr int TILE = BM * D;                                  // elements; rows unpadded, chunks swizzled
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, lse, delta
     static constexpr int P_SLOT = 64 * 32;                               // one lane = 16 bf16 = 32 bytes
-    static constexpr int P_OFF = 2 * BUF_BYTES;
+    static constexpr int NBUF = 3;                                       // tile t (P waves), t-1 (dS waves), t+1 (in flight)
+    static constexpr int P_OFF = NBUF * BUF_BYTES;
     static constexpr int MAX_QTILES = 4096;                              // Sq <= 262144 per launch
-    static constexpr int LIST_OFF = P_OFF + 4 * 2 * P_SLOT;              // 4 slices x 2 parities of P slots
+    static constexpr int LIST_OFF = P_OFF + 4 * 4 * P_SLOT;              // 4 slices x 2 parities x 2 sub-tiles of P slots
     static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;     // two tile lists (ushort) + counts
 };
 
@@ -689,6 +692,30 @@ __device__ __forceinline__ void bwd_p_gemm_s(const __bf16 *Qs, const bf16x8 (&kr
     for (int kb = 0; kb < NK; kb++) {
         if (kb + 2 < NK) qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + (((2 * (kb + 2)) ^ sw) << 3));
         s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], s, 0, 0, 0);
+    }
+}
+
+// S (P wave, B operand K) or dP (dS wave, B operand V) of both 32-row sub-tiles of a tile: the two
+// accumulation chains alternate so no MFMA waits for its predecessor
+template <int D>
+__device__ __forceinline__ void bwd_gemm_rows2(const __bf16 *T, const bf16x8 (&breg)[D / 16], const f32x16 &zero16, int l32,
+                                               int hh, f32x16 &ra, f32x16 &rb) {
+    constexpr int NK = D / 16;
+    const __bf16 *rowa = T + l32 * D, *rowb = T + (32 + l32) * D;
+    const int swa = lds_swz<D>(l32) ^ hh, swb = lds_swz<D>(32 + l32) ^ hh;
+    ra = zero16;
+    rb = zero16;
+    bf16x8 xa[2], xb[2];
+    xa[0] = *(const bf16x8 *)(rowa + ((0 ^ swa) << 3));
+    xb[0] = *(const bf16x8 *)(rowb + ((0 ^ swb) << 3));
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + 1 < NK) {
+            xa[(kb + 1) & 1] = *(const bf16x8 *)(rowa + (((2 * (kb + 1)) ^ swa) << 3));
+            xb[(kb + 1) & 1] = *(const bf16x8 *)(rowb + (((2 * (kb + 1)) ^ swb) << 3));
+        }
+        ra = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[kb & 1], breg[kb], ra, 0, 0, 0);
+        rb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[kb & 1], breg[kb], rb, 0, 0, 0);
     }
 }
 
@@ -898,7 +925,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     uint4 qld[NLD], dld[NLD];
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
-    unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 2 * (L::P_SLOT / 4);
+    unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * (L::P_SLOT / 4);
 
     // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
     // live in straight-line loop bodies and the unmasked pass carries no bounds checks at all
@@ -982,70 +1009,69 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         gload(rep, qt);
         lds_store(0);
         __syncthreads();
-        // Steps are numbered over the stream of 32-row sub-tiles, one LDS barrier per step.  In step k the P
-        // wave does all its work on sub-tile k (S, P -> slot k & 1, dV) and the dS wave all its work on
-        // sub-tile k-1 (dP, dS with P from the slot filled one step earlier, dK): inside a step the two waves
-        // of a SIMD are independent, so one wave's softmax arithmetic runs under the other's MFMAs.  Slot
-        // (k & 1) is rewritten in step k+2, after the barrier that ends step k+1 in which it was read.  Tile
-        // t+1 is fetched into registers in step 2t and stored to the LDS buffer of tile t-1 in step 2t+1,
-        // after the barrier that ends step 2t, the last one that reads tile t-1.  Both roles execute
-        // 2T + 1 barriers.
-        unsigned *const slot0 = pslot_base, *const slot1 = pslot_base + L::P_SLOT / 4;
+        // One LDS barrier per 64-row tile.  In step t the P wave does all its work on tile t (S of both
+        // sub-tiles, P -> slots of parity t & 1, dV) and the dS wave all its work on tile t-1 (dP, dS with P
+        // from the slots filled one step earlier, dK): inside a step the two waves of a SIMD are independent,
+        // so one wave's softmax arithmetic runs under the other's MFMAs.  Slots of parity (t & 1) are
+        // rewritten in step t+2, after the barrier that ends step t+1 in which they were read.  Tile t+1 is
+        // fetched into registers at the start of step t and stored at its end into buffer (t+1) % 3, which
+        // held tile t-2, last read in step t-1.  Both roles execute T + 1 barriers.
         auto put_slot = [&](unsigned *slot, const PackedTile &t) {
             *(uint4 *)(slot + lane * 8) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
             *(uint4 *)(slot + lane * 8 + 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
         };
-        int par = 0;
+        int buf = 0, par = 0;
         if (p_role) {
             for (bool more = true; more;) {
                 mctx.row_base = qt * BM;
                 more = advance(rep, qt);
                 if (more) gload(rep, qt);
-                const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
+                const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
                 const __bf16 *dOs = Qs + L::TILE;
                 const float *lse_s = (const float *)(dOs + L::TILE);
-                f32x16 s;
-                PackedTile pp;
-                bwd_p_gemm_s<D>(Qs, kvreg, zero16, 0, l32, hh, s);
-                bwd_p_softmax<MASK>(s, lse_s, 0, hh, c2, mctx, pp);
-                put_slot(slot0, pp);
-                bwd_p_phase2<D>(dOs, acc, 0, lane, pp);
-                lds_barrier();
-                bwd_p_gemm_s<D>(Qs, kvreg, zero16, 32, l32, hh, s);
-                bwd_p_softmax<MASK>(s, lse_s, 32, hh, c2, mctx, pp);
-                put_slot(slot1, pp);
-                bwd_p_phase2<D>(dOs, acc, 32, lane, pp);
-                if (more) lds_store(par ^ 1);
+                unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
+                f32x16 sa, sb;
+                PackedTile ppa, ppb;
+                bwd_gemm_rows2<D>(Qs, kvreg, zero16, l32, hh, sa, sb);
+                bwd_p_softmax<MASK>(sa, lse_s, 0, hh, c2, mctx, ppa);
+                put_slot(slots, ppa);
+                bwd_p_softmax<MASK>(sb, lse_s, 32, hh, c2, mctx, ppb);
+                put_slot(slots + L::P_SLOT / 4, ppb);
+                bwd_p_phase2<D>(dOs, acc, 0, lane, ppa);
+                bwd_p_phase2<D>(dOs, acc, 32, lane, ppb);
+                buf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                if (more) lds_store(buf);
                 lds_barrier();
                 par ^= 1;
             }
-            lds_barrier();                         // step 2T: only the dS waves have work
+            lds_barrier();                         // step T: only the dS waves have work
         } else {
             bool more = advance(rep, qt);          // step 0: staging duties only
-            if (more) gload(rep, qt);
+            if (more) {
+                gload(rep, qt);
+                lds_store(1);
+            }
             lds_barrier();
             for (;;) {
-                const __bf16 *Qs = (const __bf16 *)(smem + par * L::BUF_BYTES);
-                const __bf16 *dOs = Qs + L::TILE;
-                const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
-                f32x16 dp;
-                PackedTile ds;
-                // step 2t+1: sub-tile 0 of tile t
-                bwd_ds_phase1<D>(dOs, kvreg, zero16, 0, l32, hh, dp);
-                bwd_ds_softmax(dlt_s, slot0, dp, 0, lane, hh, ds);
-                bwd_ds_gemm_dk<D>(Qs, acc, 0, lane, ds);
-                if (more) lds_store(par ^ 1);
-                lds_barrier();
-                // step 2t+2: sub-tile 1 of tile t; fetch tile t+2
                 const bool had_next = more;
                 if (more) {
                     more = advance(rep, qt);
                     if (more) gload(rep, qt);
                 }
-                bwd_ds_phase1<D>(dOs, kvreg, zero16, 32, l32, hh, dp);
-                bwd_ds_softmax(dlt_s, slot1, dp, 32, lane, hh, ds);
-                bwd_ds_gemm_dk<D>(Qs, acc, 32, lane, ds);
+                const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
+                const __bf16 *dOs = Qs + L::TILE;
+                const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
+                const unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
+                f32x16 dpa, dpb;
+                PackedTile dsa, dsb;
+                bwd_gemm_rows2<D>(dOs, kvreg, zero16, l32, hh, dpa, dpb);
+                bwd_ds_softmax(dlt_s, slots, dpa, 0, lane, hh, dsa);
+                bwd_ds_softmax(dlt_s, slots + L::P_SLOT / 4, dpb, 32, lane, hh, dsb);
+                bwd_ds_gemm_dk<D>(Qs, acc, 0, lane, dsa);
+                bwd_ds_gemm_dk<D>(Qs, acc, 32, lane, dsb);
+                if (more) lds_store(buf + 2 >= L::NBUF ? buf + 2 - L::NBUF : buf + 2);
                 lds_barrier();
+                buf = buf == L::NBUF - 1 ? 0 : buf + 1;
                 par ^= 1;
                 if (!had_next) break;
             }
