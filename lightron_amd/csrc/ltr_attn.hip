@@ -228,8 +228,8 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     constexpr int VS = D + 32;   // V tile row stride: transpose reads only (row + 64 B is conflict-free for them)
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int NLD = BN * CPR / 256;
-    __shared__ __attribute__((aligned(16))) __bf16 Ks[BN * KS];
-    __shared__ __attribute__((aligned(16))) __bf16 Vs[BN * VS];
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers
+    constexpr int BUF_ELEMS = BN * (KS + VS);
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -346,17 +346,26 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         }
     };
 
-    bool have = c < p.n_chunks;
-    if (have) gload(t);
-    while (have) {
-        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
-        __syncthreads();
+    // Double-buffered LDS, one LDS-only barrier per tile: the tile fetched into registers during the compute
+    // of tile t is stored into the other buffer, whose readers all passed the previous barrier.
+    auto lds_store = [&](int buf) {
+        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + BN * KS;
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            *(uint4 *)(Ks + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
-            *(uint4 *)(Vs + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
+            *(uint4 *)(Kd + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
+            *(uint4 *)(Vd + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
         }
-        __syncthreads();
+    };
+    bool have = c < p.n_chunks;
+    if (have) {
+        gload(t);
+        lds_store(0);
+    }
+    __syncthreads();
+    int par = 0;
+    while (have) {
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
+        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + BN * KS;
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
@@ -437,6 +446,9 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
             }
         }
+        if (have_next) lds_store(par ^ 1);
+        lds_barrier();
+        par ^= 1;
         have = have_next;
     }
 
@@ -1108,8 +1120,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     constexpr int VS = D + 8;    // V tile: 128-bit operand reads only (row + 16 B)
     constexpr int CPR = D / 8;
     constexpr int NLD = BN * CPR / 256;
-    __shared__ __attribute__((aligned(16))) __bf16 Ks[BN * KS];
-    __shared__ __attribute__((aligned(16))) __bf16 Vs[BN * VS];
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers
+    constexpr int BUF_ELEMS = BN * (KS + VS);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1219,17 +1231,26 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
         }
     };
 
-    bool have = c < p.n_chunks;
-    if (have) gload(t);
-    while (have) {
-        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
-        __syncthreads();
+    // Double-buffered LDS, one LDS-only barrier per tile: the tile fetched into registers during the compute
+    // of tile t is stored into the other buffer, whose readers all passed the previous barrier.
+    auto lds_store = [&](int buf) {
+        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + BN * KS;
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            *(uint4 *)(Ks + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
-            *(uint4 *)(Vs + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
+            *(uint4 *)(Kd + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
+            *(uint4 *)(Vd + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
         }
-        __syncthreads();
+    };
+    bool have = c < p.n_chunks;
+    if (have) {
+        gload(t);
+        lds_store(0);
+    }
+    __syncthreads();
+    int par = 0;
+    while (have) {
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
+        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + BN * KS;
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
@@ -1279,6 +1300,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
                 }
             }
         }
+        if (have_next) lds_store(par ^ 1);
+        lds_barrier();
+        par ^= 1;
         have = have_next;
     }
 
@@ -1314,13 +1338,26 @@ int check_device() {
 }
 
 // kernels that need more than 64 KB of dynamic LDS must opt in once per process
+template <int D>
+constexpr int fwd_lds_bytes() { return 2 * 64 * ((D + 8) + (D + 32)) * 2; }
+template <int D>
+constexpr int dq_lds_bytes() { return 2 * 64 * ((D + 24) + (D + 8)) * 2; }
+
 int enable_large_lds() {
     static int done = 0;  // 0 not yet, 1 ok, -1 failed
     if (done == 0) {
         bool ok = hipFuncSetAttribute((const void *)bwd_dkdv_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       BwdLds<128>::TOTAL) == hipSuccess &&
                   hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      BwdLds<64>::TOTAL) == hipSuccess;
+                                      BwdLds<64>::TOTAL) == hipSuccess &&
+                  hipFuncSetAttribute((const void *)fwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      fwd_lds_bytes<128>()) == hipSuccess &&
+                  hipFuncSetAttribute((const void *)fwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      fwd_lds_bytes<64>()) == hipSuccess &&
+                  hipFuncSetAttribute((const void *)bwd_dq_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      dq_lds_bytes<128>()) == hipSuccess &&
+                  hipFuncSetAttribute((const void *)bwd_dq_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      dq_lds_bytes<64>()) == hipSuccess;
         done = ok ? 1 : -1;
     }
     return done == 1 ? LTR_OK : LTR_ELAUNCH;
@@ -1410,8 +1447,10 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
         p.n_qtiles = (p.Sq + 127) / 128;
         const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
         if (nblk > 0x7fffffffLL) return LTR_EINVAL;
-        if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), 0, st, p);
+        rc = enable_large_lds();
+        if (rc) return rc;
+        if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), fwd_lds_bytes<128>(), st, p);
+        else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), fwd_lds_bytes<64>(), st, p);
     } else {
         p.n_qtiles = (p.Sq + 63) / 64;
         const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
@@ -1527,10 +1566,10 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
     if (a->D == 128) {
         if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
-        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
+        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), dq_lds_bytes<128>(), st, p);
     } else {
         if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
-        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), 0, st, p);
+        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), dq_lds_bytes<64>(), st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
