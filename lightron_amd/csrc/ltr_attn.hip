@@ -187,6 +187,16 @@ __device__ __forceinline__ bf16x8 lds_operand_tr_swz(const __bf16 *tile, int k0,
     return u.v;
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_ptr + 16*l (lds_ptr is
+// wave-uniform).  No staging registers, no LDS store pass.
+__device__ __forceinline__ void global_to_lds_b128(const void *gptr, void *lds_ptr_uniform) {
+    __builtin_amdgcn_global_load_lds(gptr, (__attribute__((address_space(3))) void *)lds_ptr_uniform, 16, 0, 0);
+}
+
+__device__ __forceinline__ void tile_barrier() {   // all outstanding tile transfers and LDS traffic, then the block barrier
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) {
     union { uint4 u; bf16x8 v; } c;
     c.u = x;
@@ -224,14 +234,15 @@ __device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
 template <int D>
 __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     constexpr int BM = 128, BN = 64;
-    constexpr int KS = D + 8;    // K tile row stride (elements): natural 128-bit operand reads
-    constexpr int VS = D + 32;   // V tile row stride: transpose reads only (row + 64 B is conflict-free for them)
     constexpr int CPR = D / 8;   // 16-byte chunks per row
-    constexpr int NLD = BN * CPR / 256;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers
-    constexpr int BUF_ELEMS = BN * (KS + VS);
+    constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
+    constexpr int NI = BN / (RPI * 4);       // such loads per wave, per tensor and per tile
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers,
+    constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
+    constexpr int BUF_ELEMS = 2 * TILE;
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hh = lane >> 5;
     const bool causal = p.flags & LTR_CAUSAL;
 
@@ -314,72 +325,53 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
     };
     settle();
 
-    const int ld_r = tid / CPR, ld_c = tid % CPR;
-    constexpr int RPL = 256 / CPR;
-    const unsigned kvo = (unsigned)(ld_r * (int)p.ks[1] + ld_c * 8), vvo = (unsigned)(ld_r * (int)p.vs[1] + ld_c * 8);
-    uint4 kld[NLD], vld[NLD];
+    // Tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane, no staging
+    // registers): wave w fills rows RPI*(NI*w + i) .. of the tile with its i-th load, lane l the chunk
+    // position l % CPR of row l / CPR, fetching the logical chunk that the swizzle places there.  Rows past
+    // the end of a chunk are fetched from its last row; their keys are masked.
+    const int st_row = lane / CPR, st_pc = lane % CPR;
     int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
-    auto gload = [&](int ti) {
-        const int sk = ld_sk;
+    auto gload = [&](int ti, int buf) {
         nx_sk = ld_sk;
         nx_pos0 = ld_pos0;
         nx_key0 = ti * BN;
-        const __bf16 *kp = ld_kb + (long long)(ti * BN * (int)p.ks[1]);
-        const __bf16 *vp = ld_vb + (long long)(ti * BN * (int)p.vs[1]);
-        if (ti * BN + BN <= sk) {
+        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + TILE;
 #pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                kld[i] = *(const uint4 *)(kp + (kvo + (unsigned)(i * RPL * (int)p.ks[1])));
-                vld[i] = *(const uint4 *)(vp + (vvo + (unsigned)(i * RPL * (int)p.vs[1])));
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                const bool ok = ti * BN + ld_r + i * RPL < sk;   // the tile's first key always exists
-                kld[i] = *(const uint4 *)(kp + (ok ? kvo + (unsigned)(i * RPL * (int)p.ks[1]) : 0u));
-                vld[i] = *(const uint4 *)(vp + (ok ? vvo + (unsigned)(i * RPL * (int)p.vs[1]) : 0u));
-                if (!ok) {
-                    kld[i] = make_uint4(0, 0, 0, 0);
-                    vld[i] = make_uint4(0, 0, 0, 0);
-                }
-            }
+        for (int i = 0; i < NI; i++) {
+            const int row = RPI * (NI * w + i) + st_row;
+            const int key = min(ti * BN + row, ld_sk - 1);
+            const int chunk = st_pc ^ lds_swz<D>(row);
+            const __bf16 *ksrc = ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8);
+            const __bf16 *vsrc = ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8);
+            global_to_lds_b128(ksrc, Kd + RPI * (NI * w + i) * D);
+            global_to_lds_b128(vsrc, Vd + RPI * (NI * w + i) * D);
         }
     };
 
-    // Double-buffered LDS, one LDS-only barrier per tile: the tile fetched into registers during the compute
-    // of tile t is stored into the other buffer, whose readers all passed the previous barrier.
-    auto lds_store = [&](int buf) {
-        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + BN * KS;
-#pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            *(uint4 *)(Kd + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
-            *(uint4 *)(Vd + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
-        }
-    };
+    // Double-buffered LDS, one barrier per tile: tile t+1 streams into the other buffer (whose readers all
+    // passed the previous barrier) while tile t is computed; the barrier also waits for those loads.
     bool have = c < p.n_chunks;
-    if (have) {
-        gload(t);
-        lds_store(0);
-    }
-    __syncthreads();
+    if (have) gload(t, 0);
+    tile_barrier();
     int par = 0;
     while (have) {
         const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
-        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + BN * KS;
+        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + TILE;
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
-        if (have_next) gload(t);
+        if (have_next) gload(t, par ^ 1);
 
         // the two key blocks accumulate in alternation: a dependent MFMA cannot issue until its predecessor
         // has left the pipe, so every chain needs an independent one to fill the gap
         f32x16 s[2];
         s[0] = zero16;
         s[1] = zero16;
+        const int sw0 = lds_swz<D>(l32) ^ hh, sw1 = lds_swz<D>(32 + l32) ^ hh;   // chunk 2*kb + hh lives at (2*kb) ^ sw
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
-            const bf16x8 a0 = *(const bf16x8 *)(Ks + l32 * KS + kb * 16 + 8 * hh);
-            const bf16x8 a1 = *(const bf16x8 *)(Ks + (32 + l32) * KS + kb * 16 + 8 * hh);
+            const bf16x8 a0 = *(const bf16x8 *)(Ks + l32 * D + (((2 * kb) ^ sw0) << 3));
+            const bf16x8 a1 = *(const bf16x8 *)(Ks + (32 + l32) * D + (((2 * kb) ^ sw1) << 3));
             s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qreg[kb], s[0], 0, 0, 0);
             s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qreg[kb], s[1], 0, 0, 0);
         }
@@ -442,12 +434,11 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
             const bf16x8 pb = operand_of(pt[kb >> 1], kb & 1);
 #pragma unroll
             for (int db = 0; db < D / 32; db++) {
-                bf16x8 a = lds_operand_tr(Vs, VS, kb * 16, db * 32, lane);
+                bf16x8 a = lds_operand_tr_swz<D>(Vs, kb * 16, db * 32, lane);
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
             }
         }
-        if (have_next) lds_store(par ^ 1);
-        lds_barrier();
+        tile_barrier();
         par ^= 1;
         have = have_next;
     }
@@ -1116,12 +1107,12 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
 template <int D>
 __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     constexpr int BM = 128, BN = 64;
-    constexpr int KS = D + 24;   // K tile: 128-bit operand reads and transpose reads (row + 48 B)
-    constexpr int VS = D + 8;    // V tile: 128-bit operand reads only (row + 16 B)
     constexpr int CPR = D / 8;
-    constexpr int NLD = BN * CPR / 256;
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers
-    constexpr int BUF_ELEMS = BN * (KS + VS);
+    constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
+    constexpr int NI = BN / (RPI * 4);       // such loads per wave, per tensor and per tile
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers,
+    constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
+    constexpr int BUF_ELEMS = 2 * TILE;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1200,61 +1191,36 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     };
     settle();
 
-    const int ld_r = tid / CPR, ld_c = tid % CPR;
-    constexpr int RPL = 256 / CPR;
-    uint4 kld[NLD], vld[NLD];
+    // Tiles go from global memory straight into LDS (see the forward kernel): wave w fills rows
+    // RPI*(NI*w + i) .. with its i-th load; rows past the end of a chunk repeat its last row and are masked.
+    const int st_row = lane / CPR, st_pc = lane % CPR;
     int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
-    auto gload = [&](int ti) {
-        const int sk = ld_sk;
+    auto gload = [&](int ti, int buf) {
         nx_sk = ld_sk;
         nx_pos0 = ld_pos0;
         nx_key0 = ti * BN;
-        const __bf16 *kp = ld_kb + (long long)(ti * BN * (int)p.ks[1]);
-        const __bf16 *vp = ld_vb + (long long)(ti * BN * (int)p.vs[1]);
-        const unsigned kvo = (unsigned)(ld_r * (int)p.ks[1] + ld_c * 8), vvo = (unsigned)(ld_r * (int)p.vs[1] + ld_c * 8);
-        if (ti * BN + BN <= sk) {
+        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + TILE;
 #pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                kld[i] = *(const uint4 *)(kp + (kvo + (unsigned)(i * RPL * (int)p.ks[1])));
-                vld[i] = *(const uint4 *)(vp + (vvo + (unsigned)(i * RPL * (int)p.vs[1])));
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                kld[i] = make_uint4(0, 0, 0, 0);
-                vld[i] = make_uint4(0, 0, 0, 0);
-                if (ti * BN + ld_r + i * RPL < sk) {
-                    kld[i] = *(const uint4 *)(kp + (kvo + (unsigned)(i * RPL * (int)p.ks[1])));
-                    vld[i] = *(const uint4 *)(vp + (vvo + (unsigned)(i * RPL * (int)p.vs[1])));
-                }
-            }
+        for (int i = 0; i < NI; i++) {
+            const int row = RPI * (NI * w + i) + st_row;
+            const int key = min(ti * BN + row, ld_sk - 1);
+            const int chunk = st_pc ^ lds_swz<D>(row);
+            global_to_lds_b128(ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8), Kd + RPI * (NI * w + i) * D);
+            global_to_lds_b128(ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8), Vd + RPI * (NI * w + i) * D);
         }
     };
 
-    // Double-buffered LDS, one LDS-only barrier per tile: the tile fetched into registers during the compute
-    // of tile t is stored into the other buffer, whose readers all passed the previous barrier.
-    auto lds_store = [&](int buf) {
-        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + BN * KS;
-#pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            *(uint4 *)(Kd + (ld_r + i * RPL) * KS + ld_c * 8) = kld[i];
-            *(uint4 *)(Vd + (ld_r + i * RPL) * VS + ld_c * 8) = vld[i];
-        }
-    };
     bool have = c < p.n_chunks;
-    if (have) {
-        gload(t);
-        lds_store(0);
-    }
-    __syncthreads();
+    if (have) gload(t, 0);
+    tile_barrier();
     int par = 0;
     while (have) {
         const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
-        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + BN * KS;
+        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + TILE;
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
-        if (have_next) gload(t);
+        if (have_next) gload(t, par ^ 1);
 
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         // two 32-key halves one after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
@@ -1262,10 +1228,11 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
             f32x16 s = zero16, dp = zero16;
+            const int sw = lds_swz<D>(nb * 32 + l32) ^ hh;       // chunk 2*kb + hh lives at (2*kb) ^ sw
 #pragma unroll
             for (int kb = 0; kb < D / 16; kb++) {
-                const bf16x8 ak = *(const bf16x8 *)(Ks + (nb * 32 + l32) * KS + kb * 16 + 8 * hh);
-                const bf16x8 av = *(const bf16x8 *)(Vs + (nb * 32 + l32) * VS + kb * 16 + 8 * hh);
+                const bf16x8 ak = *(const bf16x8 *)(Ks + (nb * 32 + l32) * D + (((2 * kb) ^ sw) << 3));
+                const bf16x8 av = *(const bf16x8 *)(Vs + (nb * 32 + l32) * D + (((2 * kb) ^ sw) << 3));
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ak, qreg[kb], s, 0, 0, 0);
                 dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, doreg[kb], dp, 0, 0, 0);
             }
@@ -1295,13 +1262,12 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
                 const bf16x8 dsb = operand_of(ds, kb);
 #pragma unroll
                 for (int db = 0; db < D / 32; db++) {
-                    const bf16x8 a = lds_operand_tr(Ks, KS, nb * 32 + kb * 16, db * 32, lane);
+                    const bf16x8 a = lds_operand_tr_swz<D>(Ks, nb * 32 + kb * 16, db * 32, lane);
                     dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsb, dqacc[db], 0, 0, 0);
                 }
             }
         }
-        if (have_next) lds_store(par ^ 1);
-        lds_barrier();
+        tile_barrier();
         par ^= 1;
         have = have_next;
     }
@@ -1339,9 +1305,9 @@ int check_device() {
 
 // kernels that need more than 64 KB of dynamic LDS must opt in once per process
 template <int D>
-constexpr int fwd_lds_bytes() { return 2 * 64 * ((D + 8) + (D + 32)) * 2; }
+constexpr int fwd_lds_bytes() { return 2 * 2 * 64 * D * 2; }
 template <int D>
-constexpr int dq_lds_bytes() { return 2 * 64 * ((D + 24) + (D + 8)) * 2; }
+constexpr int dq_lds_bytes() { return 2 * 2 * 64 * D * 2; }
 
 int enable_large_lds() {
     static int done = 0;  // 0 not yet, 1 ok, -1 failed
