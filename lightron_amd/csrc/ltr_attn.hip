@@ -823,8 +823,8 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     using L = BwdLds<D>;
     constexpr int BN = L::BN, BM = L::BM, NT = L::NT;
     constexpr int CPR = D / 8;
-    constexpr int NLD = BM * CPR / NT;   // 16-byte chunks per thread per tile and tensor (2 for D=128, 1 for D=64)
-    constexpr int RPL = NT / CPR;        // rows covered by one pass of the block's threads
+    constexpr int RPI = 64 / CPR;        // rows filled by one wave-wide LDS-direct load (1 KB)
+    constexpr int NI = BM / (RPI * 8);   // such loads per wave, per tensor and per tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -920,12 +920,8 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     }
     __syncthreads();
 
-    // per-thread staging coordinates: row (tid / CPR) + RPL*i, 16-byte chunk tid % CPR
-    const int ld_r = tid / CPR, ld_c = tid % CPR;
-    const unsigned q_voff = (unsigned)(ld_r * (int)p.qs[1] + ld_c * 8);
-    const unsigned do_voff = (unsigned)(ld_r * (int)p.dos[1] + ld_c * 8);
+    const int st_row = lane / CPR, st_pc = lane % CPR;   // this lane's place inside a 1 KB LDS-direct load
     const float st_mul = tid < BM ? LTR_LOG2E : 1.f;  // threads 0..63 stage LSE*log2e, 64..127 stage DELTA
-    uint4 qld[NLD], dld[NLD];
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
     unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * (L::P_SLOT / 4);
@@ -946,49 +942,38 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             qt = __builtin_amdgcn_readfirstlane((int)list[li_]);
             return true;
         };
-        auto gload = [&](int rep, int qt) {
+        // Q and dO tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane): wave w
+        // fills rows RPI*(NI*w + i) .. of both tiles with its i-th pair of loads, lane l the chunk position
+        // l % CPR of row l / CPR, fetching the logical chunk the swizzle places there.  Rows past the end of Q
+        // repeat its last row (they are masked).  LSE and DELTA go through a register of threads 0..127.
+        auto gload = [&](int rep, int qt, int buf) {
             const int h = hkv * p.n_rep + rep;
             const int row0 = qt * BM;
-            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2] + (long long)(row0 * (int)p.qs[1]);
-            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2] + (long long)(row0 * (int)p.dos[1]);
+            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
+            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
             const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
             const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
-            if (!MASK) {
+            __bf16 *Qd = (__bf16 *)(smem + buf * L::BUF_BYTES), *dOd = Qd + L::TILE;
 #pragma unroll
-                for (int i = 0; i < NLD; i++) {
-                    qld[i] = *(const uint4 *)(qp + (q_voff + (unsigned)(i * RPL * (int)p.qs[1])));
-                    dld[i] = *(const uint4 *)(dop + (do_voff + (unsigned)(i * RPL * (int)p.dos[1])));
-                }
-                if (tid < 2 * BM) sld = sp[tid];
-            } else {
-#pragma unroll
-                for (int i = 0; i < NLD; i++) {
-                    const bool ok = row0 + ld_r + i * RPL < p.Sq;
-                    const unsigned qo = ok ? q_voff + (unsigned)(i * RPL * (int)p.qs[1]) : 0u;
-                    const unsigned dO = ok ? do_voff + (unsigned)(i * RPL * (int)p.dos[1]) : 0u;
-                    qld[i] = *(const uint4 *)(qp + qo);     // row0 itself is always a valid row
-                    dld[i] = *(const uint4 *)(dop + dO);
-                    if (!ok) {
-                        qld[i] = make_uint4(0, 0, 0, 0);
-                        dld[i] = make_uint4(0, 0, 0, 0);
-                    }
-                }
-                if (tid < 2 * BM) {
+            for (int i = 0; i < NI; i++) {
+                const int row = RPI * (NI * w + i) + st_row;
+                const int grow = MASK ? min(row0 + row, p.Sq - 1) : row0 + row;
+                const int chunk = st_pc ^ lds_swz<D>(row);
+                global_to_lds_b128(qp + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D);
+                global_to_lds_b128(dop + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D);
+            }
+            if (tid < 2 * BM) {
+                if (!MASK) {
+                    sld = sp[tid];
+                } else {
                     const int r = tid < BM ? tid : tid - BM;
                     sld_ok = row0 + r < p.Sq;
                     sld = sp[sld_ok ? tid : (tid < BM ? 0 : BM)];
                 }
             }
         };
-        auto lds_store = [&](int buf) {
-            __bf16 *Qs = (__bf16 *)(smem + buf * L::BUF_BYTES);
-            __bf16 *dOs = Qs + L::TILE;
-            float *st = (float *)(dOs + L::TILE);
-#pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                *(uint4 *)(Qs + lds_swz_off<D>(ld_r + i * RPL, ld_c)) = qld[i];
-                *(uint4 *)(dOs + lds_swz_off<D>(ld_r + i * RPL, ld_c)) = dld[i];
-            }
+        auto lds_store = [&](int buf) {   // the LSE / DELTA values fetched by gload
+            float *st = (float *)(smem + buf * L::BUF_BYTES) + L::TILE;   // after the two bf16 tiles
             if (tid < 2 * BM) {
                 float x = sld * st_mul;
                 // rows past the end: LSE = +inf makes P = 0 (they are masked as well)
@@ -1009,9 +994,9 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         int rep = 0, qt = 0;
         advance(rep, qt);
         __syncthreads();   // the previous pass has finished reading LDS
-        gload(rep, qt);
+        gload(rep, qt, 0);
         lds_store(0);
-        __syncthreads();
+        tile_barrier();
         // One LDS barrier per 64-row tile.  In step t the P wave does all its work on tile t (S of both
         // sub-tiles, P -> slots of parity t & 1, dV) and the dS wave all its work on tile t-1 (dP, dS with P
         // from the slots filled one step earlier, dK): inside a step the two waves of a SIMD are independent,
@@ -1028,7 +1013,8 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             for (bool more = true; more;) {
                 mctx.row_base = qt * BM;
                 more = advance(rep, qt);
-                if (more) gload(rep, qt);
+                const int nbuf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                if (more) gload(rep, qt, nbuf);
                 const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
                 const __bf16 *dOs = Qs + L::TILE;
                 const float *lse_s = (const float *)(dOs + L::TILE);
@@ -1042,24 +1028,21 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 put_slot(slots + L::P_SLOT / 4, ppb);
                 bwd_p_phase2<D>(dOs, acc, 0, lane, ppa);
                 bwd_p_phase2<D>(dOs, acc, 32, lane, ppb);
-                buf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                buf = nbuf;
                 if (more) lds_store(buf);
-                lds_barrier();
+                tile_barrier();
                 par ^= 1;
             }
-            lds_barrier();                         // step T: only the dS waves have work
+            tile_barrier();                        // step T: only the dS waves have work
         } else {
             bool more = advance(rep, qt);          // step 0: staging duties only
-            if (more) {
-                gload(rep, qt);
-                lds_store(1);
-            }
-            lds_barrier();
+            if (more) gload(rep, qt, 1);
+            tile_barrier();
             for (;;) {
                 const bool had_next = more;
                 if (more) {
                     more = advance(rep, qt);
-                    if (more) gload(rep, qt);
+                    if (more) gload(rep, qt, buf + 2 >= L::NBUF ? buf + 2 - L::NBUF : buf + 2);
                 }
                 const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
                 const __bf16 *dOs = Qs + L::TILE;
@@ -1072,8 +1055,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 bwd_ds_softmax(dlt_s, slots + L::P_SLOT / 4, dpb, 32, lane, hh, dsb);
                 bwd_ds_gemm_dk<D>(Qs, acc, 0, lane, dsa);
                 bwd_ds_gemm_dk<D>(Qs, acc, 32, lane, dsb);
-                if (more) lds_store(buf + 2 >= L::NBUF ? buf + 2 - L::NBUF : buf + 2);
-                lds_barrier();
+                tile_barrier();
                 buf = buf == L::NBUF - 1 ? 0 : buf + 1;
                 par ^= 1;
                 if (!had_next) break;
