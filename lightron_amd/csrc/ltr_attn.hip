@@ -5,17 +5,24 @@
 //   fwd_bf16_kernel<D>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a wave
 //                        owns 32 query rows, so a lane owns ONE query: the row max / sum are
 //                        in-lane reductions plus one v_permlane32_swap, and P^T leaves the
-//                        first GEMM already in the B-operand layout of the second.  K and V
-//                        tiles are staged in LDS by 128-bit loads; the V^T operand is read
-//                        with ds_read_b64_tr_b16.  The (O, LSE) merge with an earlier partial
-//                        result is part of the epilogue.
+//                        first GEMM already in the B-operand layout of the second.  64-key K
+//                        and V tiles go global -> LDS directly (no staging registers) into
+//                        unpadded, XOR-swizzled, double-buffered tiles, one barrier per tile;
+//                        the V^T operand is read with ds_read_b64_tr_b16.  The (O, LSE) merge
+//                        with an earlier partial result is part of the epilogue.
 //   fwd_f32_kernel<D>    fp32 I/O and arithmetic (no MFMA), for the 1e-4 parity case.
 //   delta_kernel         DELTA = rowsum(dO * O).
-//   bwd_dkdv_kernel<D>   a block owns 128 keys of one kv head (32 per wave, K and V operands
-//                        resident in registers), loops over the query heads of the GQA group
-//                        and over query tiles; dK^T/dV^T accumulate in registers.
-//   bwd_dq_kernel<D>     forward-shaped: a block owns 128 query rows, loops over K/V tiles,
-//                        dQ^T accumulates in registers.  No atomics anywhere: results are
+//   bwd_dkdv_kernel<D>   a block of 8 waves owns 128 keys of one kv head and loops over the
+//                        query heads of the GQA group and over 64-row query tiles taken from
+//                        lists (fully visible / partly masked) built once in LDS.  Two waves
+//                        share each 32-key slice: one computes S, P and dV^T, the other dP,
+//                        dS and dK^T one tile behind, P handed over through LDS.  Q / dO tiles
+//                        go global -> LDS directly into three swizzled buffers, one barrier
+//                        per tile; K, V operands and the dK^T / dV^T accumulators stay in
+//                        registers for the whole block.
+//   bwd_dq_kernel<D>     forward-shaped: a block owns 128 query rows, loops over K/V tiles
+//                        (same direct-to-LDS tiles as the forward), recomputes S and dP and
+//                        accumulates dQ^T in registers.  No atomics anywhere: results are
 //                        bitwise reproducible.
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, i = l % 32, h = l / 32):
