@@ -154,13 +154,6 @@ __device__ __forceinline__ bf16x8 lds_operand_tr(const __bf16 *tile, int stride,
     return u.v;
 }
 
-// Block barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global
-// load (workgroup-scope fence), which would expose the latency of the tile prefetch that is meant to
-// stay in flight across the barrier.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 // Unpadded row-major LDS tile of D bf16 per row whose 16-byte chunks are XOR-swizzled: chunk c of row r
 // lives at chunk position c ^ lds_swz<D>(r).  LDS has 64 banks of 4 bytes; a 128-bit read is served 16
 // lanes at a time and a 64-bit (transpose) read 32 lanes at a time.  With this permutation both the MFMA
@@ -194,14 +187,28 @@ __device__ __forceinline__ bf16x8 lds_operand_tr_swz(const __bf16 *tile, int k0,
     return u.v;
 }
 
-// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_ptr + 16*l (lds_ptr is
-// wave-uniform).  No staging registers, no LDS store pass.
-__device__ __forceinline__ void global_to_lds_b128(const void *gptr, void *lds_ptr_uniform) {
-    __builtin_amdgcn_global_load_lds(gptr, (__attribute__((address_space(3))) void *)lds_ptr_uniform, 16, 0, 0);
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at LDS byte address lds_byte_addr + 16*l
+// (wave-uniform; lds_address() of a __shared__ object plus an offset).  No staging registers, no LDS store pass.  Written as inline assembly so that the compiler
+// does not track the transfer: with the builtin it makes the next LDS read of ANY address wait for vmcnt(0),
+// which would expose the whole global-memory latency in the middle of a tile.  The transfer is only complete
+// after tile_barrier() (the only place that waits for it); nothing may read the destination before that.
+__device__ __forceinline__ unsigned lds_address(const void *shared_object) {
+    return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const void *)shared_object;
 }
 
-__device__ __forceinline__ void tile_barrier() {   // all outstanding tile transfers and LDS traffic, then the block barrier
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+__device__ __forceinline__ void global_to_lds_b128(const void *gptr, unsigned lds_byte_addr_uniform) {
+    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr_uniform);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
+// End of a tile: wait for every outstanding tile transfer and LDS access of this wave, then the block
+// barrier.  The wait is the s_waitcnt builtin (vmcnt(0) lgkmcnt(0), expcnt left alone) so that the compiler's
+// own counter bookkeeping knows that nothing is pending afterwards.
+__device__ __forceinline__ void tile_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) {
@@ -342,7 +349,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         nx_sk = ld_sk;
         nx_pos0 = ld_pos0;
         nx_key0 = ti * BN;
-        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + TILE;
+        const unsigned Kd = lds_address(smem) + buf * BUF_ELEMS * 2, Vd = Kd + TILE * 2;   // LDS byte addresses
 #pragma unroll
         for (int i = 0; i < NI; i++) {
             const int row = RPI * (NI * w + i) + st_row;
@@ -350,8 +357,8 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
             const int chunk = st_pc ^ lds_swz<D>(row);
             const __bf16 *ksrc = ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8);
             const __bf16 *vsrc = ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8);
-            global_to_lds_b128(ksrc, Kd + RPI * (NI * w + i) * D);
-            global_to_lds_b128(vsrc, Vd + RPI * (NI * w + i) * D);
+            global_to_lds_b128(ksrc, Kd + RPI * (NI * w + i) * D * 2);
+            global_to_lds_b128(vsrc, Vd + RPI * (NI * w + i) * D * 2);
         }
     };
 
@@ -960,14 +967,14 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
             const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
             const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
-            __bf16 *Qd = (__bf16 *)(smem + buf * L::BUF_BYTES), *dOd = Qd + L::TILE;
+            const unsigned Qd = lds_address(smem) + buf * L::BUF_BYTES, dOd = Qd + L::TILE * 2;   // LDS byte addresses
 #pragma unroll
             for (int i = 0; i < NI; i++) {
                 const int row = RPI * (NI * w + i) + st_row;
                 const int grow = MASK ? min(row0 + row, p.Sq - 1) : row0 + row;
                 const int chunk = st_pc ^ lds_swz<D>(row);
-                global_to_lds_b128(qp + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D);
-                global_to_lds_b128(dop + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D);
+                global_to_lds_b128(qp + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D * 2);
+                global_to_lds_b128(dop + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D * 2);
             }
             if (tid < 2 * BM) {
                 if (!MASK) {
@@ -1188,14 +1195,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
         nx_sk = ld_sk;
         nx_pos0 = ld_pos0;
         nx_key0 = ti * BN;
-        __bf16 *Kd = (__bf16 *)smem + buf * BUF_ELEMS, *Vd = Kd + TILE;
+        const unsigned Kd = lds_address(smem) + buf * BUF_ELEMS * 2, Vd = Kd + TILE * 2;   // LDS byte addresses
 #pragma unroll
         for (int i = 0; i < NI; i++) {
             const int row = RPI * (NI * w + i) + st_row;
             const int key = min(ti * BN + row, ld_sk - 1);
             const int chunk = st_pc ^ lds_swz<D>(row);
-            global_to_lds_b128(ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8), Kd + RPI * (NI * w + i) * D);
-            global_to_lds_b128(ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8), Vd + RPI * (NI * w + i) * D);
+            global_to_lds_b128(ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8), Kd + RPI * (NI * w + i) * D * 2);
+            global_to_lds_b128(ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8), Vd + RPI * (NI * w + i) * D * 2);
         }
     };
 
