@@ -244,6 +244,37 @@ __device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
     return c.v;
 }
 
+// Two independent 32x32 accumulation chains over the head dimension, A operands from rows of swizzled LDS tiles
+// (row pointers rowa / rowb, swizzle words swa / swb of those rows, already XOR-ed with the lane's half),
+// B operands from registers.  The chains alternate so no MFMA waits for its predecessor, and the operand reads
+// run PF steps ahead of the MFMAs that use them; sched_barrier pins that order (left alone, the scheduler sinks
+// each read to just before its use and the full LDS latency is exposed at every step).
+template <int D>
+__device__ __forceinline__ void lds_gemm_pair(const __bf16 *rowa, int swa, const __bf16 *rowb, int swb,
+                                              const bf16x8 (&ba)[D / 16], const bf16x8 (&bb)[D / 16],
+                                              const f32x16 &zero16, f32x16 &ra, f32x16 &rb) {
+    constexpr int NK = D / 16, PF = 2;
+    bf16x8 xa[PF + 1], xb[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        xa[i] = *(const bf16x8 *)(rowa + (((2 * i) ^ swa) << 3));
+        xb[i] = *(const bf16x8 *)(rowb + (((2 * i) ^ swb) << 3));
+    }
+    ra = zero16;
+    rb = zero16;
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + PF < NK) {
+            xa[(kb + PF) % (PF + 1)] = *(const bf16x8 *)(rowa + (((2 * (kb + PF)) ^ swa) << 3));
+            xb[(kb + PF) % (PF + 1)] = *(const bf16x8 *)(rowb + (((2 * (kb + PF)) ^ swb) << 3));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        ra = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[kb % (PF + 1)], ba[kb], ra, 0, 0, 0);
+        rb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[kb % (PF + 1)], bb[kb], rb, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // ------------------------------------------------------------------------------ forward, bf16
 template <int D>
 __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
@@ -376,19 +407,10 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         const bool have_next = c < p.n_chunks;
         if (have_next) gload(t, par ^ 1);
 
-        // the two key blocks accumulate in alternation: a dependent MFMA cannot issue until its predecessor
-        // has left the pipe, so every chain needs an independent one to fill the gap
+        // S^T of the two 32-key blocks of the tile
         f32x16 s[2];
-        s[0] = zero16;
-        s[1] = zero16;
-        const int sw0 = lds_swz<D>(l32) ^ hh, sw1 = lds_swz<D>(32 + l32) ^ hh;   // chunk 2*kb + hh lives at (2*kb) ^ sw
-#pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) {
-            const bf16x8 a0 = *(const bf16x8 *)(Ks + l32 * D + (((2 * kb) ^ sw0) << 3));
-            const bf16x8 a1 = *(const bf16x8 *)(Ks + (32 + l32) * D + (((2 * kb) ^ sw1) << 3));
-            s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qreg[kb], s[0], 0, 0, 0);
-            s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qreg[kb], s[1], 0, 0, 0);
-        }
+        lds_gemm_pair<D>(Ks + l32 * D, lds_swz<D>(l32) ^ hh, Ks + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, qreg, qreg,
+                         zero16, s[0], s[1]);
         // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         if (need_mask) {
@@ -712,28 +734,11 @@ __device__ __forceinline__ void bwd_p_gemm_s(const __bf16 *Qs, const bf16x8 (&kr
     }
 }
 
-// S (P wave, B operand K) or dP (dS wave, B operand V) of both 32-row sub-tiles of a tile: the two
-// accumulation chains alternate so no MFMA waits for its predecessor
+// S (P wave, B operand K) or dP (dS wave, B operand V) of both 32-row sub-tiles of a tile
 template <int D>
 __device__ __forceinline__ void bwd_gemm_rows2(const __bf16 *T, const bf16x8 (&breg)[D / 16], const f32x16 &zero16, int l32,
                                                int hh, f32x16 &ra, f32x16 &rb) {
-    constexpr int NK = D / 16;
-    const __bf16 *rowa = T + l32 * D, *rowb = T + (32 + l32) * D;
-    const int swa = lds_swz<D>(l32) ^ hh, swb = lds_swz<D>(32 + l32) ^ hh;
-    ra = zero16;
-    rb = zero16;
-    bf16x8 xa[2], xb[2];
-    xa[0] = *(const bf16x8 *)(rowa + ((0 ^ swa) << 3));
-    xb[0] = *(const bf16x8 *)(rowb + ((0 ^ swb) << 3));
-#pragma unroll
-    for (int kb = 0; kb < NK; kb++) {
-        if (kb + 1 < NK) {
-            xa[(kb + 1) & 1] = *(const bf16x8 *)(rowa + (((2 * (kb + 1)) ^ swa) << 3));
-            xb[(kb + 1) & 1] = *(const bf16x8 *)(rowb + (((2 * (kb + 1)) ^ swb) << 3));
-        }
-        ra = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[kb & 1], breg[kb], ra, 0, 0, 0);
-        rb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[kb & 1], breg[kb], rb, 0, 0, 0);
-    }
+    lds_gemm_pair<D>(T + l32 * D, lds_swz<D>(l32) ^ hh, T + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, breg, breg, zero16, ra, rb);
 }
 
 // P wave: P = exp2(S*c2 - LSE*log2e) -> packed bf16 in accumulator layout
@@ -1223,15 +1228,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
         // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
-            f32x16 s = zero16, dp = zero16;
+            f32x16 s, dp;
             const int sw = lds_swz<D>(nb * 32 + l32) ^ hh;       // chunk 2*kb + hh lives at (2*kb) ^ sw
-#pragma unroll
-            for (int kb = 0; kb < D / 16; kb++) {
-                const bf16x8 ak = *(const bf16x8 *)(Ks + (nb * 32 + l32) * D + (((2 * kb) ^ sw) << 3));
-                const bf16x8 av = *(const bf16x8 *)(Vs + (nb * 32 + l32) * D + (((2 * kb) ^ sw) << 3));
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ak, qreg[kb], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, doreg[kb], dp, 0, 0, 0);
-            }
+            lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, sw, Vs + (nb * 32 + l32) * D, sw, qreg, doreg, zero16, s, dp);
             PackedTile ds;
 #pragma unroll
             for (int j = 0; j < 8; j++) {
