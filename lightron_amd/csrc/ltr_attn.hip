@@ -277,11 +277,11 @@ __device__ __forceinline__ void lds_gemm_pair(const __bf16 *rowa, int swa, const
 
 // ------------------------------------------------------------------------------ forward, bf16
 template <int D>
-__global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
-    constexpr int BM = 128, BN = 64;
+__global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
+    constexpr int NW = 8, BM = 32 * NW, BN = 64;   // 8 waves (two per SIMD) share every K / V tile
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
-    constexpr int NI = BN / (RPI * 4);       // such loads per wave, per tensor and per tile
+    constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers,
     constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
     constexpr int BUF_ELEMS = 2 * TILE;
@@ -407,10 +407,13 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
         const bool have_next = c < p.n_chunks;
         if (have_next) gload(t, par ^ 1);
 
-        // S^T of the two 32-key blocks of the tile
+        // S^T of the two 32-key blocks of the tile.  The wave raises its priority while it issues MFMAs: the
+        // other wave of the SIMD then fills the gaps with its softmax arithmetic instead of delaying them.
+        __builtin_amdgcn_s_setprio(1);
         f32x16 s[2];
         lds_gemm_pair<D>(Ks + l32 * D, lds_swz<D>(l32) ^ hh, Ks + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, qreg, qreg,
                          zero16, s[0], s[1]);
+        __builtin_amdgcn_s_setprio(0);
         // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         if (need_mask) {
@@ -465,6 +468,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
                 l_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_run, false);   // sums the rounded P that PV uses
                 pt[nb].u[j] = __builtin_bit_cast(unsigned, pr);
             }
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
             const bf16x8 pb = operand_of(pt[kb >> 1], kb & 1);
@@ -474,6 +478,7 @@ __global__ __launch_bounds__(256, 2) void fwd_bf16_kernel(const FwdParams p) {
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         tile_barrier();
         par ^= 1;
         have = have_next;
@@ -1106,11 +1111,11 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
 // per-lane scalars.  S^T = K Q^T and dP^T = V dO^T with K, V tiles natural in LDS; dS^T leaves the
 // registers as the B operand of dQ^T += K^T dS^T, whose A operand is the K tile read by transpose loads.
 template <int D>
-__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
-    constexpr int BM = 128, BN = 64;
+__global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
+    constexpr int NW = 8, BM = 32 * NW, BN = 64;   // 8 waves (two per SIMD) share every K / V tile
     constexpr int CPR = D / 8;
     constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
-    constexpr int NI = BN / (RPI * 4);       // such loads per wave, per tensor and per tile
+    constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers,
     constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
     constexpr int BUF_ELEMS = 2 * TILE;
@@ -1230,7 +1235,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
         for (int nb = 0; nb < 2; nb++) {
             f32x16 s, dp;
             const int sw = lds_swz<D>(nb * 32 + l32) ^ hh;       // chunk 2*kb + hh lives at (2*kb) ^ sw
+            __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
             lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, sw, Vs + (nb * 32 + l32) * D, sw, qreg, doreg, zero16, s, dp);
+            __builtin_amdgcn_s_setprio(0);
             PackedTile ds;
 #pragma unroll
             for (int j = 0; j < 8; j++) {
@@ -1252,6 +1259,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
                 }
                 ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
             }
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {  // 16 keys per MFMA
                 const bf16x8 dsb = operand_of(ds, kb);
@@ -1261,6 +1269,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
                     dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsb, dqacc[db], 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
         }
         tile_barrier();
         par ^= 1;
@@ -1405,13 +1414,13 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     p.n_chunks = a->n_chunks;
     hipStream_t st = (hipStream_t)stream;
     if (a->io_dtype == LTR_BF16) {
-        p.n_qtiles = (p.Sq + 127) / 128;
+        p.n_qtiles = (p.Sq + 255) / 256;
         const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
         if (nblk > 0x7fffffffLL) return LTR_EINVAL;
         rc = enable_large_lds();
         if (rc) return rc;
-        if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(256), fwd_lds_bytes<128>(), st, p);
-        else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(256), fwd_lds_bytes<64>(), st, p);
+        if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<128>(), st, p);
+        else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<64>(), st, p);
     } else {
         p.n_qtiles = (p.Sq + 63) / 64;
         const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
@@ -1523,14 +1532,14 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     rc = enable_large_lds();
     if (rc) return rc;
-    const long long nblk_q = (long long)((p.Sq + 127) / 128) * p.B * p.Hq;
+    const long long nblk_q = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
     if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
     if (a->D == 128) {
         if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
-        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(256), dq_lds_bytes<128>(), st, p);
+        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
     } else {
         if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
-        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(256), dq_lds_bytes<64>(), st, p);
+        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
