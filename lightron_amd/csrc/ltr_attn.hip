@@ -275,6 +275,26 @@ __device__ __forceinline__ void lds_gemm_pair(const __bf16 *rowa, int swa, const
     }
 }
 
+// acc[db] (32 x 32 tiles over the head dimension) += T^T-operand x B for NKB blocks of 16 tile rows starting at
+// row0: the A operands are transpose reads of the swizzled LDS tile T (rows = contraction index), the B
+// operands b[kb] come from registers.  Reads run PF MFMAs ahead, order pinned as in lds_gemm_pair.
+template <int D, int NKB>
+__device__ __forceinline__ void lds_tr_gemm(const __bf16 *T, int row0, int lane, const bf16x8 (&b)[NKB],
+                                            f32x16 (&acc)[D / 32]) {
+    constexpr int ND = D / 32, N = NKB * ND, PF = 3;
+    bf16x8 a[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF && i < N; i++) a[i] = lds_operand_tr_swz<D>(T, row0 + (i / ND) * 16, (i % ND) * 32, lane);
+#pragma unroll
+    for (int step = 0; step < N; step++) {
+        if (step + PF < N)
+            a[(step + PF) % (PF + 1)] = lds_operand_tr_swz<D>(T, row0 + ((step + PF) / ND) * 16, ((step + PF) % ND) * 32, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[step / ND], acc[step % ND], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // ------------------------------------------------------------------------------ forward, bf16
 template <int D>
 __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
@@ -376,27 +396,31 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     // the end of a chunk are fetched from its last row; their keys are masked.
     const int st_row = lane / CPR, st_pc = lane % CPR;
     int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
-    auto gload = [&](int ti, int buf) {
+    // transfer j of the tile in flight (ti, into buffer buf): j < NI are this wave's K rows, the rest its V rows
+    auto gload_one = [&](int j, int ti, int buf) {
+        const int i = j % NI;
+        const unsigned dst = lds_address(smem) + buf * BUF_ELEMS * 2 + (j / NI) * TILE * 2 + RPI * (NI * w + i) * D * 2;
+        const int row = RPI * (NI * w + i) + st_row;
+        const int key = min(ti * BN + row, ld_sk - 1);
+        const int chunk = st_pc ^ lds_swz<D>(row);
+        const __bf16 *src = j < NI ? ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8)
+                                   : ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8);
+        global_to_lds_b128(src, dst);
+    };
+    auto gload_begin = [&](int ti) {   // scalar state of the tile whose transfers are issued next
         nx_sk = ld_sk;
         nx_pos0 = ld_pos0;
         nx_key0 = ti * BN;
-        const unsigned Kd = lds_address(smem) + buf * BUF_ELEMS * 2, Vd = Kd + TILE * 2;   // LDS byte addresses
-#pragma unroll
-        for (int i = 0; i < NI; i++) {
-            const int row = RPI * (NI * w + i) + st_row;
-            const int key = min(ti * BN + row, ld_sk - 1);
-            const int chunk = st_pc ^ lds_swz<D>(row);
-            const __bf16 *ksrc = ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8);
-            const __bf16 *vsrc = ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8);
-            global_to_lds_b128(ksrc, Kd + RPI * (NI * w + i) * D * 2);
-            global_to_lds_b128(vsrc, Vd + RPI * (NI * w + i) * D * 2);
-        }
     };
 
     // Double-buffered LDS, one barrier per tile: tile t+1 streams into the other buffer (whose readers all
     // passed the previous barrier) while tile t is computed; the barrier also waits for those loads.
     bool have = c < p.n_chunks;
-    if (have) gload(t, 0);
+    if (have) {
+        gload_begin(t);
+#pragma unroll
+        for (int j = 0; j < 2 * NI; j++) gload_one(j, t, 0);
+    }
     tile_barrier();
     int par = 0;
     while (have) {
@@ -405,7 +429,14 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
-        if (have_next) gload(t, par ^ 1);
+        // All transfers of the next tile are issued here, right after the barrier: the memory pipe takes them
+        // at 64 bytes per clock and a wave waits at the issue port meanwhile; issued between MFMAs instead
+        // (measured) the same waits cost more, because they then stall waves that are feeding the matrix pipe.
+        if (have_next) {
+            gload_begin(t);
+#pragma unroll
+            for (int j = 0; j < 2 * NI; j++) gload_one(j, t, par ^ 1);
+        }
 
         // S^T of the two 32-key blocks of the tile.  The wave raises its priority while it issues MFMAs: the
         // other wave of the SIMD then fills the gaps with its softmax arithmetic instead of delaying them.
@@ -469,14 +500,9 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
                 pt[nb].u[j] = __builtin_bit_cast(unsigned, pr);
             }
         __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++) {  // 16 keys per MFMA
-            const bf16x8 pb = operand_of(pt[kb >> 1], kb & 1);
-#pragma unroll
-            for (int db = 0; db < D / 32; db++) {
-                bf16x8 a = lds_operand_tr_swz<D>(Vs, kb * 16, db * 32, lane);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, oacc[db], 0, 0, 0);
-            }
+        {
+            const bf16x8 pb[4] = {operand_of(pt[0], 0), operand_of(pt[0], 1), operand_of(pt[1], 0), operand_of(pt[1], 1)};
+            lds_tr_gemm<D, 4>(Vs, 0, lane, pb, oacc);   // 16 keys per MFMA
         }
         __builtin_amdgcn_s_setprio(0);
         tile_barrier();
@@ -721,24 +747,6 @@ __device__ __forceinline__ bool bwd_visible(const BwdMaskCtx &m, int r0, int r, 
     return m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
 }
 
-// P wave: S = Q K^T for rows r0..r0+31 of the tile
-template <int D>
-__device__ __forceinline__ void bwd_p_gemm_s(const __bf16 *Qs, const bf16x8 (&kreg)[D / 16], const f32x16 &zero16, int r0,
-                                             int l32, int hh, f32x16 &s) {
-    constexpr int NK = D / 16;
-    const __bf16 *qrow = Qs + (r0 + l32) * D;
-    const int sw = lds_swz<D>(r0 + l32) ^ hh;           // chunk 2*kb + hh lives at (2*kb) ^ sw
-    s = zero16;
-    bf16x8 qb[3];
-    qb[0] = *(const bf16x8 *)(qrow + ((0 ^ sw) << 3));
-    qb[1] = *(const bf16x8 *)(qrow + ((2 ^ sw) << 3));
-#pragma unroll
-    for (int kb = 0; kb < NK; kb++) {
-        if (kb + 2 < NK) qb[(kb + 2) % 3] = *(const bf16x8 *)(qrow + (((2 * (kb + 2)) ^ sw) << 3));
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qb[kb % 3], kreg[kb], s, 0, 0, 0);
-    }
-}
-
 // S (P wave, B operand K) or dP (dS wave, B operand V) of both 32-row sub-tiles of a tile
 template <int D>
 __device__ __forceinline__ void bwd_gemm_rows2(const __bf16 *T, const bf16x8 (&breg)[D / 16], const f32x16 &zero16, int l32,
@@ -764,44 +772,6 @@ __device__ __forceinline__ void bwd_p_softmax(const f32x16 &s, const float *lse_
     }
 }
 
-// P wave, second half: dV^T += dO^T P
-template <int D>
-__device__ __forceinline__ void bwd_p_phase2(const __bf16 *dOs, f32x16 (&dvacc)[D / 32], int r0, int lane,
-                                             const PackedTile &pp) {
-    constexpr int ND = D / 32;
-    bf16x8 ao = lds_operand_tr_swz<D>(dOs, r0, 0, lane);
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-        const bf16x8 pop = operand_of(pp, kb);
-#pragma unroll
-        for (int db = 0; db < ND; db++) {
-            const int step = kb * ND + db;
-            bf16x8 aon = ao;
-            if (step + 1 < 2 * ND) aon = lds_operand_tr_swz<D>(dOs, r0 + ((step + 1) / ND) * 16, ((step + 1) % ND) * 32, lane);
-            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ao, pop, dvacc[db], 0, 0, 0);
-            ao = aon;
-        }
-    }
-}
-
-// dS wave, first half: dP = dO V^T
-template <int D>
-__device__ __forceinline__ void bwd_ds_phase1(const __bf16 *dOs, const bf16x8 (&vreg)[D / 16], const f32x16 &zero16, int r0,
-                                              int l32, int hh, f32x16 &dp) {
-    constexpr int NK = D / 16;
-    const __bf16 *drow = dOs + (r0 + l32) * D;
-    const int sw = lds_swz<D>(r0 + l32) ^ hh;
-    dp = zero16;
-    bf16x8 db_[3];
-    db_[0] = *(const bf16x8 *)(drow + ((0 ^ sw) << 3));
-    db_[1] = *(const bf16x8 *)(drow + ((2 ^ sw) << 3));
-#pragma unroll
-    for (int kb = 0; kb < NK; kb++) {
-        if (kb + 2 < NK) db_[(kb + 2) % 3] = *(const bf16x8 *)(drow + (((2 * (kb + 2)) ^ sw) << 3));
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(db_[kb % 3], vreg[kb], dp, 0, 0, 0);
-    }
-}
-
 // dS wave: dS = P * (dP - DELTA) with P from the partner's LDS slot -> packed bf16
 __device__ __forceinline__ void bwd_ds_softmax(const float *dlt_s, const unsigned *pslot, const f32x16 &dp, int r0, int lane,
                                                int hh, PackedTile &ds) {
@@ -819,26 +789,6 @@ __device__ __forceinline__ void bwd_ds_softmax(const float *dlt_s, const unsigne
         }
         ds.u[2 * g] = pack2_bf16(dsv[0], dsv[1]);
         ds.u[2 * g + 1] = pack2_bf16(dsv[2], dsv[3]);
-    }
-}
-
-// dS wave: dK^T += Q^T dS
-template <int D>
-__device__ __forceinline__ void bwd_ds_gemm_dk(const __bf16 *Qs, f32x16 (&dkacc)[D / 32], int r0, int lane,
-                                               const PackedTile &ds) {
-    constexpr int ND = D / 32;
-    bf16x8 aq = lds_operand_tr_swz<D>(Qs, r0, 0, lane);
-#pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
-        const bf16x8 dsop = operand_of(ds, kb);
-#pragma unroll
-        for (int db = 0; db < ND; db++) {
-            const int step = kb * ND + db;
-            bf16x8 aqn = aq;
-            if (step + 1 < 2 * ND) aqn = lds_operand_tr_swz<D>(Qs, r0 + ((step + 1) / ND) * 16, ((step + 1) % ND) * 32, lane);
-            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq, dsop, dkacc[db], 0, 0, 0);
-            aq = aqn;
-        }
     }
 }
 
@@ -1045,13 +995,19 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
                 f32x16 sa, sb;
                 PackedTile ppa, ppb;
+                __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
                 bwd_gemm_rows2<D>(Qs, kvreg, zero16, l32, hh, sa, sb);
+                __builtin_amdgcn_s_setprio(0);
                 bwd_p_softmax<MASK>(sa, lse_s, 0, hh, c2, mctx, ppa);
                 put_slot(slots, ppa);
                 bwd_p_softmax<MASK>(sb, lse_s, 32, hh, c2, mctx, ppb);
                 put_slot(slots + L::P_SLOT / 4, ppb);
-                bwd_p_phase2<D>(dOs, acc, 0, lane, ppa);
-                bwd_p_phase2<D>(dOs, acc, 32, lane, ppb);
+                __builtin_amdgcn_s_setprio(1);
+                {   // dV^T += dO^T P over the 64 rows of the tile
+                    const bf16x8 pb[4] = {operand_of(ppa, 0), operand_of(ppa, 1), operand_of(ppb, 0), operand_of(ppb, 1)};
+                    lds_tr_gemm<D, 4>(dOs, 0, lane, pb, acc);
+                }
+                __builtin_amdgcn_s_setprio(0);
                 buf = nbuf;
                 if (more) lds_store(buf);
                 tile_barrier();
@@ -1074,11 +1030,17 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 const unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
                 f32x16 dpa, dpb;
                 PackedTile dsa, dsb;
+                __builtin_amdgcn_s_setprio(1);
                 bwd_gemm_rows2<D>(dOs, kvreg, zero16, l32, hh, dpa, dpb);
+                __builtin_amdgcn_s_setprio(0);
                 bwd_ds_softmax(dlt_s, slots, dpa, 0, lane, hh, dsa);
                 bwd_ds_softmax(dlt_s, slots + L::P_SLOT / 4, dpb, 32, lane, hh, dsb);
-                bwd_ds_gemm_dk<D>(Qs, acc, 0, lane, dsa);
-                bwd_ds_gemm_dk<D>(Qs, acc, 32, lane, dsb);
+                __builtin_amdgcn_s_setprio(1);
+                {   // dK^T += Q^T dS over the 64 rows of the tile
+                    const bf16x8 db_[4] = {operand_of(dsa, 0), operand_of(dsa, 1), operand_of(dsb, 0), operand_of(dsb, 1)};
+                    lds_tr_gemm<D, 4>(Qs, 0, lane, db_, acc);
+                }
+                __builtin_amdgcn_s_setprio(0);
                 tile_barrier();
                 buf = buf == L::NBUF - 1 ? 0 : buf + 1;
                 par ^= 1;
@@ -1260,14 +1222,9 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
                 ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
             }
             __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++) {  // 16 keys per MFMA
-                const bf16x8 dsb = operand_of(ds, kb);
-#pragma unroll
-                for (int db = 0; db < D / 32; db++) {
-                    const bf16x8 a = lds_operand_tr_swz<D>(Ks, nb * 32 + kb * 16, db * 32, lane);
-                    dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsb, dqacc[db], 0, 0, 0);
-                }
+            {
+                const bf16x8 dsb[2] = {operand_of(ds, 0), operand_of(ds, 1)};
+                lds_tr_gemm<D, 2>(Ks, nb * 32, lane, dsb, dqacc);   // 16 keys per MFMA
             }
             __builtin_amdgcn_s_setprio(0);
         }
