@@ -244,7 +244,7 @@ __device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
     return c.v;
 }
 
-// Two independent 32x32 accumulation chains over the head dimension, A operands from rows of swizzled LDS tiles
+// Two independent 32x32 accumulation chains over the head dimension (added to ra / rb as passed in), A operands from rows of swizzled LDS tiles
 // (row pointers rowa / rowb, swizzle words swa / swb of those rows, already XOR-ed with the lane's half),
 // B operands from registers.  The chains alternate so no MFMA waits for its predecessor, and the operand reads
 // run PF steps ahead of the MFMAs that use them; sched_barrier pins that order (left alone, the scheduler sinks
@@ -252,7 +252,7 @@ __device__ __forceinline__ bf16x8 operand_of(const PackedTile &t, int kb) {
 template <int D>
 __device__ __forceinline__ void lds_gemm_pair(const __bf16 *rowa, int swa, const __bf16 *rowb, int swb,
                                               const bf16x8 (&ba)[D / 16], const bf16x8 (&bb)[D / 16],
-                                              const f32x16 &zero16, f32x16 &ra, f32x16 &rb) {
+                                              f32x16 &ra, f32x16 &rb) {
     constexpr int NK = D / 16, PF = 2;
     bf16x8 xa[PF + 1], xb[PF + 1];
 #pragma unroll
@@ -260,8 +260,6 @@ __device__ __forceinline__ void lds_gemm_pair(const __bf16 *rowa, int swa, const
         xa[i] = *(const bf16x8 *)(rowa + (((2 * i) ^ swa) << 3));
         xb[i] = *(const bf16x8 *)(rowb + (((2 * i) ^ swb) << 3));
     }
-    ra = zero16;
-    rb = zero16;
 #pragma unroll
     for (int kb = 0; kb < NK; kb++) {
         if (kb + PF < NK) {
@@ -441,9 +439,9 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         // S^T of the two 32-key blocks of the tile.  The wave raises its priority while it issues MFMAs: the
         // other wave of the SIMD then fills the gaps with its softmax arithmetic instead of delaying them.
         __builtin_amdgcn_s_setprio(1);
-        f32x16 s[2];
+        f32x16 s[2] = {zero16, zero16};
         lds_gemm_pair<D>(Ks + l32 * D, lds_swz<D>(l32) ^ hh, Ks + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, qreg, qreg,
-                         zero16, s[0], s[1]);
+                         s[0], s[1]);
         __builtin_amdgcn_s_setprio(0);
         // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
@@ -748,10 +746,11 @@ __device__ __forceinline__ bool bwd_visible(const BwdMaskCtx &m, int r0, int r, 
 }
 
 // S (P wave, B operand K) or dP (dS wave, B operand V) of both 32-row sub-tiles of a tile
+// (added to ra / rb as passed in)
 template <int D>
-__device__ __forceinline__ void bwd_gemm_rows2(const __bf16 *T, const bf16x8 (&breg)[D / 16], const f32x16 &zero16, int l32,
-                                               int hh, f32x16 &ra, f32x16 &rb) {
-    lds_gemm_pair<D>(T + l32 * D, lds_swz<D>(l32) ^ hh, T + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, breg, breg, zero16, ra, rb);
+__device__ __forceinline__ void bwd_gemm_rows2(const __bf16 *T, const bf16x8 (&breg)[D / 16], int l32, int hh, f32x16 &ra,
+                                               f32x16 &rb) {
+    lds_gemm_pair<D>(T + l32 * D, lds_swz<D>(l32) ^ hh, T + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, breg, breg, ra, rb);
 }
 
 // P wave: P = exp2(S*c2 - LSE*log2e) -> packed bf16 in accumulator layout
@@ -772,20 +771,18 @@ __device__ __forceinline__ void bwd_p_softmax(const f32x16 &s, const float *lse_
     }
 }
 
-// dS wave: dS = P * (dP - DELTA) with P from the partner's LDS slot -> packed bf16
-__device__ __forceinline__ void bwd_ds_softmax(const float *dlt_s, const unsigned *pslot, const f32x16 &dp, int r0, int lane,
-                                               int hh, PackedTile &ds) {
-    const uint4 p0 = *(const uint4 *)(pslot + lane * 8), p1 = *(const uint4 *)(pslot + lane * 8 + 4);
+// dS wave: dS = P * (dP - DELTA) with P from the partner's LDS slot -> packed bf16; dpm = dP - DELTA
+__device__ __forceinline__ void bwd_ds_softmax(const unsigned *pslot, const f32x16 &dpm, int lane, PackedTile &ds) {
+    const uint4 p0 = *(const uint4 *)(pslot + lane * 4), p1 = *(const uint4 *)(pslot + 256 + lane * 4);
     const unsigned pu[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-        const f32x4 dv = *(const f32x4 *)(dlt_s + r0 + 8 * g + 4 * hh);
         float dsv[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const unsigned u = pu[2 * g + e / 2];
             const float pv = __uint_as_float((e & 1) ? (u & 0xffff0000u) : (u << 16));   // masked entries are 0
-            dsv[e] = pv * (dp[4 * g + e] - dv[e]);
+            dsv[e] = pv * dpm[4 * g + e];
         }
         ds.u[2 * g] = pack2_bf16(dsv[0], dsv[1]);
         ds.u[2 * g + 1] = pack2_bf16(dsv[2], dsv[3]);
@@ -895,7 +892,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     __syncthreads();
 
     const int st_row = lane / CPR, st_pc = lane % CPR;   // this lane's place inside a 1 KB LDS-direct load
-    const float st_mul = tid < BM ? LTR_LOG2E : 1.f;  // threads 0..63 stage LSE*log2e, 64..127 stage DELTA
+    const float st_mul = tid < BM ? LTR_LOG2E : -1.f;  // threads 0..63 stage LSE*log2e, 64..127 stage -DELTA
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
     unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * (L::P_SLOT / 4);
@@ -979,8 +976,9 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         // fetched into registers at the start of step t and stored at its end into buffer (t+1) % 3, which
         // held tile t-2, last read in step t-1.  Both roles execute T + 1 barriers.
         auto put_slot = [&](unsigned *slot, const PackedTile &t) {
-            *(uint4 *)(slot + lane * 8) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
-            *(uint4 *)(slot + lane * 8 + 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
+            // two 16-byte halves per lane, each half contiguous over the lanes (no bank conflicts)
+            *(uint4 *)(slot + lane * 4) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
+            *(uint4 *)(slot + 256 + lane * 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
         };
         int buf = 0, par = 0;
         if (p_role) {
@@ -993,10 +991,10 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 const __bf16 *dOs = Qs + L::TILE;
                 const float *lse_s = (const float *)(dOs + L::TILE);
                 unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
-                f32x16 sa, sb;
+                f32x16 sa = zero16, sb = zero16;
                 PackedTile ppa, ppb;
                 __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
-                bwd_gemm_rows2<D>(Qs, kvreg, zero16, l32, hh, sa, sb);
+                bwd_gemm_rows2<D>(Qs, kvreg, l32, hh, sa, sb);
                 __builtin_amdgcn_s_setprio(0);
                 bwd_p_softmax<MASK>(sa, lse_s, 0, hh, c2, mctx, ppa);
                 put_slot(slots, ppa);
@@ -1028,13 +1026,23 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 const __bf16 *dOs = Qs + L::TILE;
                 const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
                 const unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
+                // the dP accumulators start at -DELTA of their rows (register r <-> tile row 8*(r/4) + 4*hh + r%4)
                 f32x16 dpa, dpb;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 da = *(const f32x4 *)(dlt_s + 8 * g + 4 * hh), db4 = *(const f32x4 *)(dlt_s + 32 + 8 * g + 4 * hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        dpa[4 * g + e] = da[e];
+                        dpb[4 * g + e] = db4[e];
+                    }
+                }
                 PackedTile dsa, dsb;
                 __builtin_amdgcn_s_setprio(1);
-                bwd_gemm_rows2<D>(dOs, kvreg, zero16, l32, hh, dpa, dpb);
+                bwd_gemm_rows2<D>(dOs, kvreg, l32, hh, dpa, dpb);
                 __builtin_amdgcn_s_setprio(0);
-                bwd_ds_softmax(dlt_s, slots, dpa, 0, lane, hh, dsa);
-                bwd_ds_softmax(dlt_s, slots + L::P_SLOT / 4, dpb, 32, lane, hh, dsb);
+                bwd_ds_softmax(slots, dpa, lane, dsa);
+                bwd_ds_softmax(slots + L::P_SLOT / 4, dpb, lane, dsb);
                 __builtin_amdgcn_s_setprio(1);
                 {   // dK^T += Q^T dS over the 64 rows of the tile
                     const bf16x8 db_[4] = {operand_of(dsa, 0), operand_of(dsa, 1), operand_of(dsb, 0), operand_of(dsb, 1)};
@@ -1195,10 +1203,10 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
         // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
-            f32x16 s, dp;
+            f32x16 s = zero16, dp = zero16;
             const int sw = lds_swz<D>(nb * 32 + l32) ^ hh;       // chunk 2*kb + hh lives at (2*kb) ^ sw
             __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
-            lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, sw, Vs + (nb * 32 + l32) * D, sw, qreg, doreg, zero16, s, dp);
+            lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, sw, Vs + (nb * 32 + l32) * D, sw, qreg, doreg, s, dp);
             __builtin_amdgcn_s_setprio(0);
             PackedTile ds;
 #pragma unroll
