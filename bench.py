@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
 # HBM-side bytes per launch of bwd_dkdv_kernel<128> on config 3, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # command calibrated against streaming kernels of known size (profiles/bench_c3_counters.md)
-DKDV_C3_TRAFFIC_BYTES = 2.04e9
+DKDV_C3_TRAFFIC_BYTES = 2.13e9
 
 
 def _workload(name):
@@ -105,8 +105,8 @@ def _cpu_baseline(cfg, threads):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()

@@ -2,8 +2,9 @@
 // KV chunks resident in HBM, recompute backward, behind the C ABI of include/ltr_attn.h.
 //
 // Kernel map
-//   fwd_bf16_kernel<D>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a wave
-//                        owns 32 query rows, so a lane owns ONE query: the row max / sum are
+//   fwd_bf16_kernel<D>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a block of
+//                        8 waves owns 256 query rows, a wave 32 of them, so a lane owns ONE query:
+//                        the row max / sum are
 //                        in-lane reductions plus one v_permlane32_swap, and P^T leaves the
 //                        first GEMM already in the B-operand layout of the second.  64-key K
 //                        and V tiles go global -> LDS directly (no staging registers) into
@@ -20,7 +21,7 @@
 //                        go global -> LDS directly into three swizzled buffers, one barrier
 //                        per tile; K, V operands and the dK^T / dV^T accumulators stay in
 //                        registers for the whole block.
-//   bwd_dq_kernel<D>     forward-shaped: a block owns 128 query rows, loops over K/V tiles
+//   bwd_dq_kernel<D>     forward-shaped: a block owns 256 query rows, loops over K/V tiles
 //                        (same direct-to-LDS tiles as the forward), recomputes S and dP and
 //                        accumulates dQ^T in registers.  No atomics anywhere: results are
 //                        bitwise reproducible.
@@ -711,21 +712,21 @@ __global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst
 //                    the four 32-key slices one "P wave" (S = Q K^T, P, dV^T += dO^T P; K operand in
 //                    registers) and one "dS wave" (dP = dO V^T, dS = P*(dP - DELTA), dK^T += Q^T dS;
 //                    V operand in registers).  The P wave hands P (bf16, accumulator layout) to its
-//                    partner through a 2 KB LDS slot; both GEMM pairs of a 32-row sub-tile are
-//                    separated by one block barrier.  The block loops over the query heads of the
-//                    GQA group and over 64-row Q / dO tiles staged in double-buffered LDS; dK^T and
-//                    dV^T stay in registers for the whole loop.
-//   bwd_dq_kernel    a block owns 128 query rows of one query head (32 per wave; Q and dO
+//                    partner through a 2 KB LDS slot; the dS wave runs one tile behind, so one block
+//                    barrier per tile is enough.  The block loops over the query heads of the GQA
+//                    group and over 64-row Q / dO tiles in triple-buffered LDS; dK^T and dV^T stay
+//                    in registers for the whole loop.
+//   bwd_dq_kernel    a block owns 256 query rows of one query head (32 per wave; Q and dO
 //                    operands in registers), loops over 64-key K/V tiles like the forward;
 //                    dQ^T accumulates in registers.
-// LDS of bwd_dkdv_kernel (dynamic): two buffers of {Q tile, dO tile, LSE*log2e, DELTA}, then the P slots.
+// LDS of bwd_dkdv_kernel (dynamic): three buffers of {Q tile, dO tile, LSE*log2e, -DELTA}, the P slots, the tile lists.
 template <int D>
 struct BwdLds {
     static constexpr int BN = 128;      // keys per block, 32 per wave pair
     static constexpr int BM = 64;       // query rows per tile (two 32-row MFMA sub-tiles)
     static constexpr int NT = 512;      // threads per block
     static constexpr int TILE = BM * D;                                  // elements; rows unpadded, chunks swizzled
-    static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, lse, delta
+    static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, LSE*log2e, -DELTA
     static constexpr int P_SLOT = 64 * 32;                               // one lane = 16 bf16 = 32 bytes
     static constexpr int NBUF = 3;                                       // tile t (P waves), t-1 (dS waves), t+1 (in flight)
     static constexpr int P_OFF = NBUF * BUF_BYTES;
