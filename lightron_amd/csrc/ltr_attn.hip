@@ -199,7 +199,7 @@ __device__ __forceinline__ unsigned lds_address(const void *shared_object) {
 
 __device__ __forceinline__ void global_to_lds_b128(const void *gptr, unsigned lds_byte_addr_uniform) {
     const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr_uniform);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
 }
 
 // End of a tile: wait for every outstanding tile transfer and LDS access of this wave, then the block
@@ -274,12 +274,39 @@ __device__ __forceinline__ void lds_gemm_pair(const __bf16 *rowa, int swa, const
     }
 }
 
+struct NoHook {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+
+// One 32x32 accumulation chain over the head dimension (added to r as passed in): A operands from row `row` of a
+// swizzled LDS tile (sw = swizzle word of the row XOR the lane's half), B operands from registers.  hook(kb)
+// is placed right after MFMA kb: independent arithmetic of the same wave written there issues while the matrix
+// pipe works on that MFMA (a wave issues one instruction per ~5 clocks, an MFMA occupies the pipe for 32).
+template <int D, class Hook = NoHook>
+__device__ __forceinline__ void lds_gemm_chain(const __bf16 *row, int sw, const bf16x8 (&b)[D / 16], f32x16 &r,
+                                               Hook hook = Hook()) {
+    constexpr int NK = D / 16, PF = 2;
+    bf16x8 x[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF; i++) x[i] = *(const bf16x8 *)(row + (((2 * i) ^ sw) << 3));
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + PF < NK) x[(kb + PF) % (PF + 1)] = *(const bf16x8 *)(row + (((2 * (kb + PF)) ^ sw) << 3));
+        __builtin_amdgcn_sched_barrier(0);
+        r = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[kb % (PF + 1)], b[kb], r, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        hook(kb);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // acc[db] (32 x 32 tiles over the head dimension) += T^T-operand x B for NKB blocks of 16 tile rows starting at
 // row0: the A operands are transpose reads of the swizzled LDS tile T (rows = contraction index), the B
-// operands b[kb] come from registers.  Reads run PF MFMAs ahead, order pinned as in lds_gemm_pair.
-template <int D, int NKB>
+// operands b[kb] come from registers.  Reads run PF MFMAs ahead, order pinned as in lds_gemm_pair; hook(step)
+// is placed right after MFMA `step` (see lds_gemm_chain).
+template <int D, int NKB, class Hook = NoHook>
 __device__ __forceinline__ void lds_tr_gemm(const __bf16 *T, int row0, int lane, const bf16x8 (&b)[NKB],
-                                            f32x16 (&acc)[D / 32]) {
+                                            f32x16 (&acc)[D / 32], Hook hook = Hook()) {
     constexpr int ND = D / 32, N = NKB * ND, PF = 3;
     bf16x8 a[PF + 1];
 #pragma unroll
@@ -290,6 +317,8 @@ __device__ __forceinline__ void lds_tr_gemm(const __bf16 *T, int row0, int lane,
             a[(step + PF) % (PF + 1)] = lds_operand_tr_swz<D>(T, row0 + ((step + PF) / ND) * 16, ((step + PF) % ND) * 32, lane);
         __builtin_amdgcn_sched_barrier(0);
         acc[step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[step / ND], acc[step % ND], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        hook(step);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
@@ -746,48 +775,23 @@ __device__ __forceinline__ bool bwd_visible(const BwdMaskCtx &m, int r0, int r, 
     return m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
 }
 
-// S (P wave, B operand K) or dP (dS wave, B operand V) of both 32-row sub-tiles of a tile
-// (added to ra / rb as passed in)
-template <int D>
-__device__ __forceinline__ void bwd_gemm_rows2(const __bf16 *T, const bf16x8 (&breg)[D / 16], int l32, int hh, f32x16 &ra,
-                                               f32x16 &rb) {
-    lds_gemm_pair<D>(T + l32 * D, lds_swz<D>(l32) ^ hh, T + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, breg, breg, ra, rb);
-}
-
-// P wave: P = exp2(S*c2 - LSE*log2e) -> packed bf16 in accumulator layout
+// P wave, accumulator registers 2j and 2j+1 of a 32x32 sub-tile: sm = S - LSE / scale (the accumulator started at
+// -LSE / scale), P = exp2(sm * c2) -> one packed bf16 pair in accumulator layout
 template <bool MASK>
-__device__ __forceinline__ void bwd_p_softmax(const f32x16 &s, const float *lse_s, int r0, int hh, float c2,
-                                              const BwdMaskCtx &m, PackedTile &pp) {
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const f32x4 lv = *(const f32x4 *)(lse_s + r0 + 8 * g + 4 * hh);
-        float pv[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            pv[e] = __builtin_amdgcn_exp2f(s[4 * g + e] * c2 - lv[e]);
-            if (MASK) pv[e] = bwd_visible(m, r0, 4 * g + e, hh) ? pv[e] : 0.f;
-        }
-        pp.u[2 * g] = pack2_bf16(pv[0], pv[1]);
-        pp.u[2 * g + 1] = pack2_bf16(pv[2], pv[3]);
+__device__ __forceinline__ unsigned bwd_p_pair(const f32x16 &sm, int j, int r0, int hh, float c2, const BwdMaskCtx &m) {
+    float p0 = __builtin_amdgcn_exp2f(sm[2 * j] * c2), p1 = __builtin_amdgcn_exp2f(sm[2 * j + 1] * c2);
+    if (MASK) {
+        p0 = bwd_visible(m, r0, 2 * j, hh) ? p0 : 0.f;
+        p1 = bwd_visible(m, r0, 2 * j + 1, hh) ? p1 : 0.f;
     }
+    return pack2_bf16(p0, p1);
 }
 
-// dS wave: dS = P * (dP - DELTA) with P from the partner's LDS slot -> packed bf16; dpm = dP - DELTA
-__device__ __forceinline__ void bwd_ds_softmax(const unsigned *pslot, const f32x16 &dpm, int lane, PackedTile &ds) {
-    const uint4 p0 = *(const uint4 *)(pslot + lane * 4), p1 = *(const uint4 *)(pslot + 256 + lane * 4);
-    const unsigned pu[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-        float dsv[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const unsigned u = pu[2 * g + e / 2];
-            const float pv = __uint_as_float((e & 1) ? (u & 0xffff0000u) : (u << 16));   // masked entries are 0
-            dsv[e] = pv * dpm[4 * g + e];
-        }
-        ds.u[2 * g] = pack2_bf16(dsv[0], dsv[1]);
-        ds.u[2 * g + 1] = pack2_bf16(dsv[2], dsv[3]);
-    }
+// dS wave, the same pair: dS = P * (dP - DELTA), pu = packed P pair from the partner's LDS slot (masked entries
+// are 0), dpm = dP - DELTA (the accumulator started at -DELTA)
+__device__ __forceinline__ unsigned bwd_ds_pair(unsigned pu, const f32x16 &dpm, int j) {
+    const float p0 = __uint_as_float(pu << 16), p1 = __uint_as_float(pu & 0xffff0000u);
+    return pack2_bf16(p0 * dpm[2 * j], p1 * dpm[2 * j + 1]);
 }
 
 template <int D>
@@ -893,7 +897,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     __syncthreads();
 
     const int st_row = lane / CPR, st_pc = lane % CPR;   // this lane's place inside a 1 KB LDS-direct load
-    const float st_mul = tid < BM ? LTR_LOG2E : -1.f;  // threads 0..63 stage LSE*log2e, 64..127 stage -DELTA
+    const float st_mul = tid < BM ? -1.f / p.scale : -1.f;  // threads 0..63 stage -LSE/scale, 64..127 stage -DELTA
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
     unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * (L::P_SLOT / 4);
@@ -906,12 +910,15 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         const int cnt = __builtin_amdgcn_readfirstlane(tcount[cls - 1]);
         const unsigned short *const list = tlist + (cls - 1) * L::MAX_QTILES;
         int li_ = -1;                                 // index into the list
+        // the list entry of the next call is read from LDS one call ahead, so its latency is never waited for
+        unsigned short pre = list[0];
         auto advance = [&](int &rep, int &qt) {   // next tile of this class after (rep, qt); false when done
             if (++li_ >= cnt) {
                 li_ = 0;
                 if (++rep >= p.n_rep) return false;
             }
-            qt = __builtin_amdgcn_readfirstlane((int)list[li_]);
+            qt = __builtin_amdgcn_readfirstlane((int)pre);
+            pre = list[li_ + 1 < cnt ? li_ + 1 : 0];
             return true;
         };
         // Q and dO tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane): wave w
@@ -948,8 +955,8 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             float *st = (float *)(smem + buf * L::BUF_BYTES) + L::TILE;   // after the two bf16 tiles
             if (tid < 2 * BM) {
                 float x = sld * st_mul;
-                // rows past the end: LSE = +inf makes P = 0 (they are masked as well)
-                if (MASK) x = sld_ok ? x : (tid < BM ? INFINITY : 0.f);
+                // rows past the end: -LSE/scale = -inf makes P = 0 (they are masked as well)
+                if (MASK) x = sld_ok ? x : (tid < BM ? -INFINITY : 0.f);
                 st[tid] = x;
             }
         };
@@ -990,22 +997,44 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 if (more) gload(rep, qt, nbuf);
                 const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
                 const __bf16 *dOs = Qs + L::TILE;
-                const float *lse_s = (const float *)(dOs + L::TILE);
+                const float *st_s = (const float *)(dOs + L::TILE);   // -LSE/scale of the tile's rows
                 unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
-                f32x16 sa = zero16, sb = zero16;
-                PackedTile ppa, ppb;
-                __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
-                bwd_gemm_rows2<D>(Qs, kvreg, l32, hh, sa, sb);
-                __builtin_amdgcn_s_setprio(0);
-                bwd_p_softmax<MASK>(sa, lse_s, 0, hh, c2, mctx, ppa);
-                put_slot(slots, ppa);
-                bwd_p_softmax<MASK>(sb, lse_s, 32, hh, c2, mctx, ppb);
-                put_slot(slots + L::P_SLOT / 4, ppb);
-                __builtin_amdgcn_s_setprio(1);
-                {   // dV^T += dO^T P over the 64 rows of the tile
-                    const bf16x8 pb[4] = {operand_of(ppa, 0), operand_of(ppa, 1), operand_of(ppb, 0), operand_of(ppb, 1)};
-                    lds_tr_gemm<D, 4>(dOs, 0, lane, pb, acc);
+                // Accumulator register r of a sub-tile <-> tile row 8*(r/4) + 4*hh + r%4: both S accumulators start at
+                // -LSE/scale of their rows.  Order of the step: S of sub-tile a; S of sub-tile b with the
+                // exponentials of a issued under its MFMAs; first half of dV (rows of a) with the exponentials of b
+                // under its MFMAs; second half of dV.
+                f32x16 sa, sb;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 la = *(const f32x4 *)(st_s + 8 * g + 4 * hh), lb = *(const f32x4 *)(st_s + 32 + 8 * g + 4 * hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        sa[4 * g + e] = la[e];
+                        sb[4 * g + e] = lb[e];
+                    }
                 }
+                PackedTile ppa, ppb;
+                constexpr int NK = D / 16, ND = D / 32;
+                __builtin_amdgcn_s_setprio(1);
+                lds_gemm_chain<D>(Qs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, sa);
+                lds_gemm_chain<D>(Qs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, sb, [&](int kb) {
+#pragma unroll
+                    for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) ppa.u[j] = bwd_p_pair<MASK>(sa, j, 0, hh, c2, mctx);
+                });
+                put_slot(slots, ppa);
+                bf16x8 pb[4];
+                pb[0] = operand_of(ppa, 0);
+                pb[1] = operand_of(ppa, 1);
+                // the operands of the second half do not exist yet: the hook below fills ppb while the first half
+                // runs, and the loop reads pb[2], pb[3] only after that; the first half reads pb[0], pb[1]
+                lds_tr_gemm<D, 2>(dOs, 0, lane, *(const bf16x8(*)[2]) & pb[0], acc, [&](int step) {
+#pragma unroll
+                    for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) ppb.u[j] = bwd_p_pair<MASK>(sb, j, 32, hh, c2, mctx);
+                });
+                put_slot(slots + L::P_SLOT / 4, ppb);
+                pb[2] = operand_of(ppb, 0);
+                pb[3] = operand_of(ppb, 1);
+                lds_tr_gemm<D, 2>(dOs, 32, lane, *(const bf16x8(*)[2]) & pb[2], acc);
                 __builtin_amdgcn_s_setprio(0);
                 buf = nbuf;
                 if (more) lds_store(buf);
@@ -1027,7 +1056,9 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 const __bf16 *dOs = Qs + L::TILE;
                 const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
                 const unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
-                // the dP accumulators start at -DELTA of their rows (register r <-> tile row 8*(r/4) + 4*hh + r%4)
+                // the dP accumulators start at -DELTA of their rows (register r <-> tile row 8*(r/4) + 4*hh + r%4);
+                // same order as the P wave: dP of a; dP of b with dS of a under its MFMAs; first half of dK with dS of
+                // b under its MFMAs; second half of dK
                 f32x16 dpa, dpb;
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
@@ -1039,16 +1070,28 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                     }
                 }
                 PackedTile dsa, dsb;
+                constexpr int NK = D / 16, ND = D / 32;
                 __builtin_amdgcn_s_setprio(1);
-                bwd_gemm_rows2<D>(dOs, kvreg, l32, hh, dpa, dpb);
-                __builtin_amdgcn_s_setprio(0);
-                bwd_ds_softmax(slots, dpa, lane, dsa);
-                bwd_ds_softmax(slots + L::P_SLOT / 4, dpb, lane, dsb);
-                __builtin_amdgcn_s_setprio(1);
-                {   // dK^T += Q^T dS over the 64 rows of the tile
-                    const bf16x8 db_[4] = {operand_of(dsa, 0), operand_of(dsa, 1), operand_of(dsb, 0), operand_of(dsb, 1)};
-                    lds_tr_gemm<D, 4>(Qs, 0, lane, db_, acc);
-                }
+                lds_gemm_chain<D>(dOs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, dpa);
+                const uint4 pa0 = *(const uint4 *)(slots + lane * 4), pa1 = *(const uint4 *)(slots + 256 + lane * 4);
+                const unsigned pua[8] = {pa0.x, pa0.y, pa0.z, pa0.w, pa1.x, pa1.y, pa1.z, pa1.w};
+                lds_gemm_chain<D>(dOs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, dpb, [&](int kb) {
+#pragma unroll
+                    for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) dsa.u[j] = bwd_ds_pair(pua[j], dpa, j);
+                });
+                const unsigned *slot_b = slots + L::P_SLOT / 4;
+                const uint4 pb0 = *(const uint4 *)(slot_b + lane * 4), pb1 = *(const uint4 *)(slot_b + 256 + lane * 4);
+                const unsigned pub[8] = {pb0.x, pb0.y, pb0.z, pb0.w, pb1.x, pb1.y, pb1.z, pb1.w};
+                bf16x8 db_[4];
+                db_[0] = operand_of(dsa, 0);
+                db_[1] = operand_of(dsa, 1);
+                lds_tr_gemm<D, 2>(Qs, 0, lane, *(const bf16x8(*)[2]) & db_[0], acc, [&](int step) {
+#pragma unroll
+                    for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) dsb.u[j] = bwd_ds_pair(pub[j], dpb, j);
+                });
+                db_[2] = operand_of(dsb, 0);
+                db_[3] = operand_of(dsb, 1);
+                lds_tr_gemm<D, 2>(Qs, 32, lane, *(const bf16x8(*)[2]) & db_[2], acc);
                 __builtin_amdgcn_s_setprio(0);
                 tile_barrier();
                 buf = buf == L::NBUF - 1 ? 0 : buf + 1;
