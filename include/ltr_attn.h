@@ -162,6 +162,34 @@ int ltr_attn_bwd(const ltr_attn_bwd_args *args, void *stream);
 /* dst[i] = bf16(src[i]) (round to nearest even), i < n; both contiguous. */
 int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream);
 
+/*
+ * ltr_rope_apply - rotary position embedding of one tensor, the arithmetic of
+ * apply_rotary_emb (layers/layers.py:44-70): x viewed as complex numbers over ADJACENT
+ * pairs (x[2i], x[2i+1]), converted to fp32, multiplied by freqs[s][i] = (cos, sin) of
+ * angle s * theta_i, converted back to the input dtype.  The reference applies it to q
+ * and k before attention (model/model.py:183, parallel/parallel_cp.py:219); one call
+ * per tensor here.  freqs is the table of precompute_freqs_cis (layers/layers.py:18-24)
+ * as interleaved fp32 (re, im) pairs, [S][D/2][2] contiguous, row s for sequence index s
+ * of x (the caller slices the table for a chunk that starts at a global position).
+ * LTR_ROPE_CONJ multiplies by the conjugate instead: that is the gradient of the
+ * rotation (torch autograd through the complex multiply in the reference).
+ * x and out may be the same buffer.  Element strides as in ltr_attn_fwd_args.
+ */
+#define LTR_ROPE_CONJ 1u
+
+typedef struct ltr_rope_args {
+    const void *x;        /* [B, S, H, D] by strides, D contiguous */
+    void *out;            /* same shape, own strides */
+    const float *freqs;   /* [S, D/2, 2] fp32 (cos, sin) */
+    int32_t B, H, D;      /* D a multiple of 8 */
+    int64_t S;
+    int64_t x_stride[3], out_stride[3];   /* elements, for B, S, H */
+    uint32_t flags;       /* LTR_ROPE_CONJ */
+    int32_t io_dtype;     /* LTR_BF16 or LTR_F32, x and out */
+} ltr_rope_args;
+
+int ltr_rope_apply(const ltr_rope_args *args, void *stream);
+
 int ltr_abi_version(void);
 const char *ltr_strerror(int code);
 

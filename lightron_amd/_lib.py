@@ -12,7 +12,7 @@ LTR_MAX_CHUNKS = 32
 LTR_BF16, LTR_F32 = 0, 1
 LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV = 1, 2, 4, 8
 
-EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16",
+EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_abi_version", "ltr_strerror")
 
 _i64x3 = ctypes.c_int64 * 3
@@ -56,6 +56,14 @@ class BwdArgs(ctypes.Structure):
                 ("chunk", KvChunk * LTR_MAX_CHUNKS)]
 
 
+class RopeArgs(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("out", ctypes.c_void_p), ("freqs", ctypes.c_void_p),
+                ("B", ctypes.c_int32), ("H", ctypes.c_int32), ("D", ctypes.c_int32),
+                ("S", ctypes.c_int64),
+                ("x_stride", _i64x3), ("out_stride", _i64x3),
+                ("flags", ctypes.c_uint32), ("io_dtype", ctypes.c_int32)]
+
+
 _lib = None
 
 
@@ -77,6 +85,8 @@ def load():
     lib.ltr_attn_bwd.restype = ctypes.c_int
     lib.ltr_cast_f32_to_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     lib.ltr_cast_f32_to_bf16.restype = ctypes.c_int
+    lib.ltr_rope_apply.argtypes = [ctypes.POINTER(RopeArgs), ctypes.c_void_p]
+    lib.ltr_rope_apply.restype = ctypes.c_int
     lib.ltr_abi_version.argtypes = []
     lib.ltr_abi_version.restype = ctypes.c_int
     lib.ltr_strerror.argtypes = [ctypes.c_int]

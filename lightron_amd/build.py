@@ -5,12 +5,11 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SRC = os.path.join(HERE, "csrc", "ltr_attn.hip")
+SRCS = [os.path.join(HERE, "csrc", "ltr_attn.hip"), os.path.join(HERE, "csrc", "ltr_rope.hip")]
 LIB = os.path.join(HERE, "csrc", "libltr_attn.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-shared", "-fPIC", "-std=c++17",
-    "-munsafe-fp-atomics",                      # hardware global_atomic_add_f32 for the dQ accumulator
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",       # MFMA results in VGPRs: no accvgpr copies around the softmax
     "-I", os.path.join(ROOT, "include"),
@@ -21,13 +20,13 @@ def build(verbose: bool = False) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     if not os.path.exists(hipcc):
         hipcc = "hipcc"
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB, SRC]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB] + SRCS
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("hipcc failed building %s" % SRC)
+        raise RuntimeError("hipcc failed building %s" % " ".join(SRCS))
     return LIB
 
 

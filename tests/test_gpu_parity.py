@@ -254,3 +254,35 @@ def test_ulysses_module_matches_oracle(ltr):
     attn_d.forward = lambda x_, f_: called.setdefault("y", x_)
     mod = ltr.ContextParallelAttention(attn_d, Args)
     assert mod(x[0].cuda(), fc.cuda()) is called["y"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_kernel_bit_exact(ltr, dtype):
+    """ltr_rope_apply against the oracle's restatement of apply_rotary_emb (layers/layers.py:44-70): the kernel
+    rounds the four products of the complex multiply separately, as torch's fp32 complex multiply on the CPU
+    does, so forward and gradient agree bit for bit in fp32 and therefore after the cast to bf16 as well."""
+    g = torch.Generator().manual_seed(11)
+    for (B, S, H, Hk, D) in ((2, 37, 3, 3, 64), (1, 64, 8, 2, 128), (1, 5, 1, 1, 8)):
+        q = torch.randn(B, S, H, D, generator=g).to(dtype)
+        k = torch.randn(B, S, Hk, D, generator=g).to(dtype)
+        fc = orc.precompute_freqs_cis(D, S + 3)[3:]                 # a chunk that starts at position 3
+        rq, _ = orc.apply_rotary_emb(q, q, fc)
+        rk, _ = orc.apply_rotary_emb(k, k, fc)
+        qd, kd = q.cuda().requires_grad_(True), k.cuda().requires_grad_(True)
+        gq, gk = ltr.apply_rotary_emb(qd, kd, fc.cuda())
+        assert gq.dtype == dtype and torch.equal(gq.detach().cpu(), rq) and torch.equal(gk.detach().cpu(), rk)
+        # gradient = rotation by the conjugate angles; the oracle's comes from torch autograd on the CPU
+        dq_ = torch.randn(B, S, H, D, generator=g).to(dtype)
+        qc = q.clone().requires_grad_(True)
+        orc.apply_rotary_emb(qc, qc, fc)[0].backward(dq_)
+        gq.backward(dq_.cuda())
+        assert torch.equal(qd.grad.cpu(), qc.grad)
+    # strided input: a [B, H, S, D] buffer viewed as [B, S, H, D]
+    x = torch.randn(2, 4, 16, 64, generator=g).to(dtype)
+    fc = orc.precompute_freqs_cis(64, 16)
+    ref, _ = orc.apply_rotary_emb(x.transpose(1, 2), x.transpose(1, 2), fc)
+    got, _ = ltr.apply_rotary_emb(x.cuda().transpose(1, 2), x.cuda().transpose(1, 2), fc.cuda())
+    assert torch.equal(got.cpu(), ref)
+    with pytest.raises(AssertionError):
+        ltr.apply_rotary_emb(x.cuda().transpose(1, 2), x.cuda().transpose(1, 2), fc.cuda()[:8])

@@ -39,6 +39,7 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(L.FwdArgs) == 3 * 8 + 4 * 4 + 8 + 4 * 24 + 16 + 8 + 4 * 5 + 4 + 32 * 48
     assert ctypes.sizeof(L.DeltaArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
     assert ctypes.sizeof(L.BwdArgs) == 5 * 8 + 4 * 4 + 8 + 7 * 24 + 16 + 8 + 4 * 4 + 32 * 48
+    assert ctypes.sizeof(L.RopeArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
 
 
 def test_validation_without_gpu():
@@ -61,6 +62,21 @@ def test_validation_without_gpu():
     assert lib.ltr_attn_bwd(None, None) == -1 and lib.ltr_attn_bwd_delta(None, None) == -1
     assert lib.ltr_cast_f32_to_bf16(None, None, 4, None) == -1
     assert lib.ltr_cast_f32_to_bf16(4096, 4096, 0, None) == 0       # empty input is a no-op
+    assert lib.ltr_rope_apply(None, None) == -1
+    r = L.RopeArgs()
+    assert lib.ltr_rope_apply(ctypes.byref(r), None) == -1          # null pointers
+    r.x = r.out = r.freqs = 4096
+    r.B, r.H, r.D, r.S = 1, 2, 12, 4
+    assert lib.ltr_rope_apply(ctypes.byref(r), None) == -2          # head dim not a multiple of 8
+    r.D, r.io_dtype = 16, 7
+    assert lib.ltr_rope_apply(ctypes.byref(r), None) == -2          # dtype
+    r.io_dtype, r.x = 0, 4100
+    assert lib.ltr_rope_apply(ctypes.byref(r), None) == -3          # misaligned x
+    r.x = 4096
+    r.x_stride[1] = 4
+    assert lib.ltr_rope_apply(ctypes.byref(r), None) == -3          # 8-byte row stride in bf16
+    r.x_stride[1], r.S = 32, 0
+    assert lib.ltr_rope_apply(ctypes.byref(r), None) == 0           # empty input is a no-op
 
 
 def test_missing_library_fails_loudly(monkeypatch):
