@@ -102,12 +102,56 @@ def _cpu_baseline(cfg, threads):
                 "fwd + autograd bwd" if cfg["bwd"] else "fwd", t_total)}
 
 
+def _bench_rope(args):
+    """RoPE pre-pass of config 4 (q chunk of rank 15 and all of k, bf16, D=128): one launch of rope_kernel per
+    tensor.  HBM bound: algorithmic bytes = read + write of every element plus one read of the (cos, sin) rows."""
+    import torch
+    import lightron_amd as la
+    la._lib.load()
+    dev = torch.device("cuda:0")
+    B, H, D, S, Sq = 1, 8, 128, 131072, 8192
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, Sq, H, D, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(dev)
+    fc = la.precompute_freqs_cis(D, S, device=dev)
+    fq = fc[S - Sq:]
+    tq, tk = torch.view_as_real(fq).contiguous(), torch.view_as_real(fc).contiguous()
+    from lightron_amd.layers import _rope_launch
+    def step():
+        _rope_launch(q, tq, False)
+        _rope_launch(k, tk, False)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _rope_launch(k, tk, False)
+        e1.record()
+        evs.append((e0, e1))
+        _rope_launch(q, tq, False)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    k_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    k_bytes = k.numel() * 4 + tk.numel() * 4          # bf16 in + bf16 out, fp32 table rows once
+    tot_bytes = k_bytes + q.numel() * 4 + tq.numel() * 4
+    out = {"metric": "RoPE pre-pass GB/s (config 4 shapes, bf16)", "value": round(tot_bytes / dt / 1e9, 1), "unit": "GB/s",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "config 4 RoPE: q [1,8192,8,128] at positions 122880.., k [1,131072,8,128], bf16"},
+           "roofline": {"bound": "hbm", "kernel": "rope_kernel<bf16>", "achieved": round(k_bytes / (k_ms * 1e-3) / 1e9, 1),
+                        "peak": 8000.0, "unit": "GB/s", "frac": round(k_bytes / (k_ms * 1e-3) / 1e9 / 8000.0, 4), "traffic": None}}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "rope"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -116,6 +160,8 @@ def main():
     import torch
     import lightron_amd as la
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.workload == "rope":
+        return _bench_rope(args)
     la._lib.load()
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")

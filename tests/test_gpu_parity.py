@@ -286,3 +286,44 @@ def test_rope_kernel_bit_exact(ltr, dtype):
     assert torch.equal(got.cpu(), ref)
     with pytest.raises(AssertionError):
         ltr.apply_rotary_emb(x.cuda().transpose(1, 2), x.cuda().transpose(1, 2), fc.cuda()[:8])
+
+
+@pytest.mark.gpu
+def test_attention_layer_gqa(ltr):
+    """lightron_amd.Attention (model/model.py:123-202 on the HIP kernels) against the reference composition restated
+    with the oracle: projections, RoPE, repeat_kv (kv head = q head // n_rep), dense causal attention, wo; forward
+    and the gradients of the input and of every weight."""
+    class Args:
+        dim, n_heads, n_kv_heads, tp_size = 256, 4, 2, 1
+    B, S, D = 2, 96, 64
+    torch.manual_seed(3)
+    layer = ltr.Attention(Args).to(torch.bfloat16)
+    x = ((torch.rand(B, S, Args.dim) * 2 - 1) * 0.5).to(torch.bfloat16)
+    dy = ((torch.rand(B, S, Args.dim) * 2 - 1) * 0.1).to(torch.bfloat16)
+    fc = orc.precompute_freqs_cis(D, S)
+    # oracle in fp32 on the CPU from the same bf16 parameters
+    ws = {n: p.detach().float().requires_grad_(True) for n, p in layer.named_parameters()}
+    xr = x.float().requires_grad_(True)
+    q = (xr @ ws["wq.weight"].T).view(B, S, 4, D)
+    k = (xr @ ws["wk.weight"].T).view(B, S, 2, D)
+    v = (xr @ ws["wv.weight"].T).view(B, S, 2, D)
+    q, k = orc.apply_rotary_emb(q, k, fc)
+    assert torch.equal(ltr.repeat_kv(k, 2), k.repeat_interleave(2, dim=2))      # model.py:11-34
+    pos = torch.arange(S)
+    o, _ = orc.dense_attention(q, k, v, pos, pos, True)
+    y_ref = o.float().flatten(2) @ ws["wo.weight"].T
+    y_ref.backward(dy.float())
+    ld = layer.cuda()
+    xd = x.cuda().requires_grad_(True)
+    y = ld(xd, fc.cuda())
+    y.backward(dy.cuda())
+    assert y.shape == (B, S, Args.dim) and y.dtype == torch.bfloat16
+    rel = lambda a, b: ((a.float().cpu() - b).norm() / b.norm()).item()
+    assert rel(y, y_ref.detach()) < 2e-2
+    assert rel(xd.grad, xr.grad) < 5e-2
+    for n, p in ld.named_parameters():
+        assert rel(p.grad, ws[n].grad) < 5e-2, n
+    with pytest.raises(NotImplementedError):
+        class A2(Args):
+            tp_size = 2
+        ltr.Attention(A2)
