@@ -277,7 +277,8 @@ def main():
     achieved = dom_flops / (dom_ms * 1e-3) / 1e12
     prop = torch.cuda.get_device_properties(0)
     out = {
-        "metric": "ring-attn fwd+bwd causal TFLOP/s at S=32k bf16, 1 GPU; % of MFMA peak",
+        "metric": ("ring-attn fwd+bwd causal TFLOP/s at S=32k bf16, 1 GPU; % of MFMA peak" if args.workload == "c3" else
+                   "attention %s causal-adjusted TFLOP/s, 1 GPU; %% of MFMA peak" % ("fwd+bwd" if bwd else "fwd")),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
