@@ -327,3 +327,25 @@ def test_attention_layer_gqa(ltr):
         class A2(Args):
             tp_size = 2
         ltr.Attention(A2)
+
+
+@pytest.mark.gpu
+def test_against_library_sdpa_on_gpu(ltr):
+    """Independent of the oracle: the installed torch's scaled_dot_product_attention on the GPU (the routine the
+    reference itself calls, model/model.py:193-198) in fp32 on the same bf16 inputs, GQA by repeat_interleave,
+    causal; forward and all three gradients at a size the dense oracle would take minutes for."""
+    import torch.nn.functional as F
+    B, S, Hq, Hkv, D = 2, 2048, 8, 2, 128
+    g = torch.Generator().manual_seed(5)
+    q, k, v, do = (torch.randn(B, S, h, D, generator=g).to(torch.bfloat16).cuda() for h in (Hq, Hkv, Hkv, Hq))
+    qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))
+    rep = Hq // Hkv
+    o_ref = F.scaled_dot_product_attention(qr.transpose(1, 2), kr.repeat_interleave(rep, 2).transpose(1, 2),
+                                           vr.repeat_interleave(rep, 2).transpose(1, 2), is_causal=True).transpose(1, 2)
+    o_ref.backward(do.float())
+    qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o, _ = ltr.block_attention(qd, [kd], [vd], [0], 0, None, causal=True)
+    o.backward(do)
+    assert (o.float() - o_ref).abs().max().item() < 2e-2
+    rel = lambda a, b: ((a.float() - b).norm() / b.norm()).item()
+    assert rel(qd.grad, qr.grad) < 5e-2 and rel(kd.grad, kr.grad) < 5e-2 and rel(vd.grad, vr.grad) < 5e-2
