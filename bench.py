@@ -198,7 +198,8 @@ def main():
     o_all = torch.empty_like(q_all)
     lse_all = torch.empty(W, B, Hq, sl, dtype=torch.float32, device=dev)
     if bwd:
-        dq_acc = torch.empty(q_all.shape, dtype=torch.float32, device=dev)
+        # every rank's call holds all KV chunks its queries see, so the dQ kernel writes bf16 dQ itself (LTR_DQ_BF16)
+        dq_out = torch.empty(q_all.shape, dtype=torch.bfloat16, device=dev)
         dk_acc = torch.empty(k_all.shape, dtype=torch.float32, device=dev)
         dv_acc = torch.empty(v_all.shape, dtype=torch.float32, device=dev)
 
@@ -226,7 +227,7 @@ def main():
 
     def step(timed):
         if bwd:
-            dq_acc.zero_(); dk_acc.zero_(); dv_acc.zero_()
+            dk_acc.zero_(); dv_acc.zero_()
         for r in cfg["ranks"]:
             ks, vs, pos, qp, qsplit = tables[r]
             timed_call("fwd", timed, lambda: la.attn_fwd(q_all[r], ks, vs, pos, qp, qsplit, causal, out=o_all[r],
@@ -236,13 +237,13 @@ def main():
                 dks, dvs = acc_views(r, dk_acc), acc_views(r, dv_acc)
                 # the two backward kernels are enqueued by two calls so each can be timed on its own
                 timed_call("dkdv", timed, lambda: la.attn_bwd_accumulate(
-                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_acc[r], dks, dvs, qp, qsplit, causal,
+                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
                     do_dq=False))
                 timed_call("dq", timed, lambda: la.attn_bwd_accumulate(
-                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_acc[r], dks, dvs, qp, qsplit, causal,
+                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
                     do_dkdv=False))
         if bwd:
-            la.cast_to_bf16(dq_acc); la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
+            la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
 
     for _ in range(args.warmup):
         step(False)

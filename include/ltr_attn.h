@@ -47,6 +47,7 @@ extern "C" {
 #define LTR_MERGE 2u  /* forward: o/lse hold an earlier partial result; merge into it */
 #define LTR_NO_DQ 4u    /* backward: skip the dQ kernel (dq may be NULL) */
 #define LTR_NO_DKDV 8u  /* backward: skip the dK/dV kernel (chunk[].dk/dv may be NULL) */
+#define LTR_DQ_BF16 16u /* backward: dq is a bf16 tensor that RECEIVES dQ of this call (no accumulation) */
 
 /* error codes */
 #define LTR_OK 0
@@ -131,14 +132,17 @@ int ltr_attn_bwd_delta(const ltr_attn_delta_args *args, void *stream);
  * dK/dV of a GQA group sum over its Hq/Hkv query heads.  Two kernels are enqueued, one
  * for dK/dV and one for dQ (no atomics: results are bitwise reproducible); LTR_NO_DQ /
  * LTR_NO_DKDV enqueue only one of them, e.g. for a ring step where dK/dV travel with the
- * KV chunk, or to time the kernels separately.
+ * KV chunk, or to time the kernels separately.  LTR_DQ_BF16: when the chunk table of this
+ * call holds every KV chunk the queries can see, dQ is complete after the call, and dq
+ * may then be the bf16 result itself (written, not accumulated; dq_stride in bf16
+ * elements): no fp32 accumulator, no zero-fill, no final cast.
  */
 typedef struct ltr_attn_bwd_args {
     const void *q;
     const void *d_o;      /* same dtype as q */
     const float *lse;     /* [B, Hq, Sq], of the COMPLETE softmax (all chunks) */
     const float *delta;   /* [B, Hq, Sq] */
-    float *dq;            /* fp32 accumulator, by dq strides */
+    void *dq;             /* fp32 accumulator by dq strides, or the bf16 result with LTR_DQ_BF16 */
     int32_t B, Hq, Hkv, D;
     int64_t Sq;
     int64_t q_stride[3];
@@ -151,7 +155,7 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;
-    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 */
     int32_t io_dtype;     /* LTR_BF16 (the backward kernels are bf16 only) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];

@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
 LTR_ABI_VERSION = 1
 LTR_MAX_CHUNKS = 32
 LTR_BF16, LTR_F32 = 0, 1
-LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV = 1, 2, 4, 8
+LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16 = 1, 2, 4, 8, 16
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_abi_version", "ltr_strerror")

@@ -123,7 +123,9 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
                         causal=False, scale=None, do_dq=True, do_dkdv=True):
     """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
-    do_dq / do_dkdv select which of the two backward kernels are enqueued."""
+    do_dq / do_dkdv select which of the two backward kernels are enqueued.  dq_acc may instead be a bf16
+    tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
+    queries can see and fit one launch (at most 32 chunks)."""
     lib = _lib.load()
     _req(q, "q")
     _req(do, "dO")
@@ -131,10 +133,15 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     ks, vs = _norm_chunks(ks, vs)
     if not (_same_strides(dk_accs) and _same_strides(dv_accs)):
         raise RuntimeError("dk/dv accumulators must share one stride triple each")
-    for t in [dq_acc] + list(dk_accs) + list(dv_accs):
+    dq_direct = dq_acc.dtype == torch.bfloat16
+    if dq_direct and do_dq and len(ks) > _lib.LTR_MAX_CHUNKS:
+        raise RuntimeError("a bf16 dQ output needs all KV chunks in one launch (at most %d)" % _lib.LTR_MAX_CHUNKS)
+    for t in ([] if dq_direct else [dq_acc]) + list(dk_accs) + list(dv_accs):
         _req(t, "accumulator")
         if t.dtype != torch.float32:
             raise RuntimeError("gradient accumulators must be fp32")
+    if dq_direct:
+        _req(dq_acc, "dQ")
     a = _lib.BwdArgs()
     a.q, a.d_o, a.lse, a.delta, a.dq = q.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(), dq_acc.data_ptr()
     a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, ks[0].shape[2], D, Sq
@@ -144,7 +151,7 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
     a.flags = ((_lib.LTR_CAUSAL if causal else 0) | (0 if do_dq else _lib.LTR_NO_DQ)
-               | (0 if do_dkdv else _lib.LTR_NO_DKDV))
+               | (0 if do_dkdv else _lib.LTR_NO_DKDV) | (_lib.LTR_DQ_BF16 if dq_direct else 0))
     a.io_dtype = _DT[q.dtype]
     stream = _stream_ptr(q.device)
     n = len(ks)
@@ -204,11 +211,14 @@ class BlockAttentionFunction(torch.autograd.Function):
             do = do.contiguous()
         do = do.to(q.dtype)
         delta = attn_delta(o, do)
-        dq_acc = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        # one launch sees every chunk: dQ is written as bf16 by the kernel; otherwise it accumulates in fp32
+        direct = n_chunks <= _lib.LTR_MAX_CHUNKS
+        dq_acc = (torch.empty(q.shape, dtype=torch.bfloat16, device=q.device) if direct
+                  else torch.zeros(q.shape, dtype=torch.float32, device=q.device))
         dk_accs = [torch.zeros(k.shape, dtype=torch.float32, device=q.device) for k in ks]
         dv_accs = [torch.zeros(v.shape, dtype=torch.float32, device=q.device) for v in vs]
         attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale)
-        dq = cast_to_bf16(dq_acc)
+        dq = dq_acc if direct else cast_to_bf16(dq_acc)
         dks = [cast_to_bf16(x) for x in dk_accs]
         dvs = [cast_to_bf16(x) for x in dv_accs]
         return (dq, None, None, None, None, None, None, None, None, *dks, *dvs)

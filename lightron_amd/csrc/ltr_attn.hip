@@ -76,7 +76,7 @@ struct BwdParams {
     const void *d_o;
     const float *lse;
     const float *delta;
-    float *dq;
+    void *dq;          // fp32 accumulator, or bf16 result with LTR_DQ_BF16
     int B, Hq, Hkv, n_rep;
     int Sq, n_qtiles;
     long long qs[3], dos[3], dqs[3], ks[3], vs[3], dks[3], dvs[3];
@@ -1286,17 +1286,31 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     }
 
     if (row_ok) {
-        float *dqp = p.dq + b * p.dqs[0] + (long long)my_row * p.dqs[1] + h * p.dqs[2];
+        const long long off = b * p.dqs[0] + (long long)my_row * p.dqs[1] + h * p.dqs[2];
+        if (p.flags & LTR_DQ_BF16) {   // this call saw every key of these rows: store the result, no accumulator
+            __bf16 *dqp = (__bf16 *)p.dq + off;
 #pragma unroll
-        for (int db = 0; db < D / 32; db++)
+            for (int db = 0; db < D / 32; db++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d = db * 32 + 8 * g + 4 * hh;
-                f32x4 old = *(const f32x4 *)(dqp + d);
+                for (int g = 0; g < 4; g++) {
+                    bf16x4 y;
 #pragma unroll
-                for (int e = 0; e < 4; e++) old[e] += dqacc[db][4 * g + e] * p.scale;
-                *(f32x4 *)(dqp + d) = old;
-            }
+                    for (int e = 0; e < 4; e++) y[e] = (__bf16)(dqacc[db][4 * g + e] * p.scale);
+                    *(bf16x4 *)(dqp + db * 32 + 8 * g + 4 * hh) = y;
+                }
+        } else {
+            float *dqp = (float *)p.dq + off;
+#pragma unroll
+            for (int db = 0; db < D / 32; db++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int d = db * 32 + 8 * g + 4 * hh;
+                    f32x4 old = *(const f32x4 *)(dqp + d);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) old[e] += dqacc[db][4 * g + e] * p.scale;
+                    *(f32x4 *)(dqp + d) = old;
+                }
+        }
     }
 }
 
@@ -1477,7 +1491,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV)) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
@@ -1488,6 +1502,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
         return LTR_EALIGN;
     for (int i = 0; i < 3; i++)
         if (a->dq_stride[i] < 0) return LTR_EINVAL;
+    if (do_dq && !strides_ok(a->dq_stride, (a->flags & LTR_DQ_BF16) ? 2 : 4)) return LTR_EALIGN;
     if ((a->Sq + 63) / 64 > BwdLds<128>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
     if ((a->Sq + 64) * a->q_stride[1] >= 0x7fffffffLL || (a->Sq + 64) * a->do_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     BwdParams p;

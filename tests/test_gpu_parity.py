@@ -349,3 +349,25 @@ def test_against_library_sdpa_on_gpu(ltr):
     assert (o.float() - o_ref).abs().max().item() < 2e-2
     rel = lambda a, b: ((a.float() - b).norm() / b.norm()).item()
     assert rel(qd.grad, qr.grad) < 5e-2 and rel(kd.grad, kr.grad) < 5e-2 and rel(vd.grad, vr.grad) < 5e-2
+
+
+@pytest.mark.gpu
+def test_dq_written_as_bf16_equals_accumulate_then_cast(ltr):
+    """LTR_DQ_BF16 (dq receives the bf16 result of a call that holds every KV chunk) against the fp32 accumulator
+    path followed by ltr_cast_f32_to_bf16: the same value is rounded once in both, so the bits agree."""
+    g = torch.Generator().manual_seed(9)
+    B, Sq, Hq, Hkv, D = 1, 300, 4, 2, 128
+    q, do = (torch.randn(B, Sq, Hq, D, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+    kf, vf = (torch.randn(B, 300, Hkv, D, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+    ks, vs, pos0 = [kf[:, :200], kf[:, 200:]], [vf[:, :200], vf[:, 200:]], [0, 200]
+    o, lse = ltr.attn_fwd(q, ks, vs, pos0, 0, None, True)
+    delta = ltr.attn_delta(o, do)
+    dkf, dvf = (torch.zeros(kf.shape, dtype=torch.float32, device="cuda") for _ in range(2))
+    dks, dvs = [dkf[:, :200], dkf[:, 200:]], [dvf[:, :200], dvf[:, 200:]]
+    acc = torch.zeros(q.shape, dtype=torch.float32, device="cuda")
+    ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, acc, dks, dvs, 0, None, True, do_dkdv=False)
+    direct = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device="cuda")
+    ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, direct, dks, dvs, 0, None, True, do_dkdv=False)
+    assert torch.equal(direct, ltr.cast_to_bf16(acc))
+    with pytest.raises(RuntimeError):
+        ltr.attn_bwd_accumulate(q, do, lse, delta, ks * 20, vs * 20, pos0 * 20, direct, dks * 20, dvs * 20, 0, None, True)
