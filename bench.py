@@ -200,6 +200,7 @@ def main():
     if bwd:
         # every rank's call holds all KV chunks its queries see, so the dQ kernel writes bf16 dQ itself (LTR_DQ_BF16)
         dq_out = torch.empty(q_all.shape, dtype=torch.bfloat16, device=dev)
+        delta_ws = torch.empty(B, Hq, sl, dtype=torch.float32, device=dev)
         dk_acc = torch.empty(k_all.shape, dtype=torch.float32, device=dev)
         dv_acc = torch.empty(v_all.shape, dtype=torch.float32, device=dev)
 
@@ -233,15 +234,15 @@ def main():
             timed_call("fwd", timed, lambda: la.attn_fwd(q_all[r], ks, vs, pos, qp, qsplit, causal, out=o_all[r],
                                                          lse=lse_all[r]))
             if bwd:
-                delta = la.attn_delta(o_all[r], do_all[r])
                 dks, dvs = acc_views(r, dk_acc), acc_views(r, dv_acc)
-                # the two backward kernels are enqueued by two calls so each can be timed on its own
-                timed_call("dkdv", timed, lambda: la.attn_bwd_accumulate(
-                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
-                    do_dq=False))
+                # the two backward kernels are enqueued by two calls so each can be timed on its own; the dQ kernel
+                # goes first and also produces DELTA = rowsum(dO * O) for the dK/dV kernel (LTR_DELTA_FROM_O)
                 timed_call("dq", timed, lambda: la.attn_bwd_accumulate(
-                    q_all[r], do_all[r], lse_all[r], delta, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
-                    do_dkdv=False))
+                    q_all[r], do_all[r], lse_all[r], delta_ws, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
+                    do_dkdv=False, o=o_all[r]))
+                timed_call("dkdv", timed, lambda: la.attn_bwd_accumulate(
+                    q_all[r], do_all[r], lse_all[r], delta_ws, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
+                    do_dq=False))
         if bwd:
             la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
 

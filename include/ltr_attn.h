@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 1
+#define LTR_ABI_VERSION 2
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -48,6 +48,7 @@ extern "C" {
 #define LTR_NO_DQ 4u    /* backward: skip the dQ kernel (dq may be NULL) */
 #define LTR_NO_DKDV 8u  /* backward: skip the dK/dV kernel (chunk[].dk/dv may be NULL) */
 #define LTR_DQ_BF16 16u /* backward: dq is a bf16 tensor that RECEIVES dQ of this call (no accumulation) */
+#define LTR_DELTA_FROM_O 32u /* backward: delta is computed from o by the dQ kernel (and written to delta) */
 
 /* error codes */
 #define LTR_OK 0
@@ -135,13 +136,16 @@ int ltr_attn_bwd_delta(const ltr_attn_delta_args *args, void *stream);
  * KV chunk, or to time the kernels separately.  LTR_DQ_BF16: when the chunk table of this
  * call holds every KV chunk the queries can see, dQ is complete after the call, and dq
  * may then be the bf16 result itself (written, not accumulated; dq_stride in bf16
- * elements): no fp32 accumulator, no zero-fill, no final cast.
+ * elements): no fp32 accumulator, no zero-fill, no final cast.  LTR_DELTA_FROM_O: delta is
+ * an OUTPUT workspace; the dQ kernel computes DELTA = rowsum(dO * O) of its rows from o
+ * (bf16, o_stride) and stores it, and the dK/dV kernel, enqueued after it, reads it: no
+ * separate ltr_attn_bwd_delta launch.  Not combinable with LTR_NO_DQ.
  */
 typedef struct ltr_attn_bwd_args {
     const void *q;
     const void *d_o;      /* same dtype as q */
     const float *lse;     /* [B, Hq, Sq], of the COMPLETE softmax (all chunks) */
-    const float *delta;   /* [B, Hq, Sq] */
+    float *delta;         /* [B, Hq, Sq] fp32: input, or workspace written with LTR_DELTA_FROM_O */
     void *dq;             /* fp32 accumulator by dq strides, or the bf16 result with LTR_DQ_BF16 */
     int32_t B, Hq, Hkv, D;
     int64_t Sq;
@@ -155,10 +159,12 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;
-    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O */
     int32_t io_dtype;     /* LTR_BF16 (the backward kernels are bf16 only) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
+    const void *o;        /* forward output, bf16, only read with LTR_DELTA_FROM_O */
+    int64_t o_stride[3];
 } ltr_attn_bwd_args;
 
 int ltr_attn_bwd(const ltr_attn_bwd_args *args, void *stream);

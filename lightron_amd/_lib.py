@@ -7,10 +7,10 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
 
-LTR_ABI_VERSION = 1
+LTR_ABI_VERSION = 2
 LTR_MAX_CHUNKS = 32
 LTR_BF16, LTR_F32 = 0, 1
-LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16 = 1, 2, 4, 8, 16
+LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O = 1, 2, 4, 8, 16, 32
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_abi_version", "ltr_strerror")
@@ -53,7 +53,8 @@ class BwdArgs(ctypes.Structure):
                 ("q_pos0", _i64x2), ("q_split", ctypes.c_int64),
                 ("scale", ctypes.c_float), ("flags", ctypes.c_uint32),
                 ("io_dtype", ctypes.c_int32), ("n_chunks", ctypes.c_int32),
-                ("chunk", KvChunk * LTR_MAX_CHUNKS)]
+                ("chunk", KvChunk * LTR_MAX_CHUNKS),
+                ("o", ctypes.c_void_p), ("o_stride", _i64x3)]
 
 
 class RopeArgs(ctypes.Structure):

@@ -121,11 +121,13 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
-                        causal=False, scale=None, do_dq=True, do_dkdv=True):
+                        causal=False, scale=None, do_dq=True, do_dkdv=True, o=None):
     """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
     do_dq / do_dkdv select which of the two backward kernels are enqueued.  dq_acc may instead be a bf16
     tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
-    queries can see and fit one launch (at most 32 chunks)."""
+    queries can see and fit one launch (at most 32 chunks).  With o (the bf16 forward output) given, delta is a
+    workspace: the dQ kernel of the first launch computes rowsum(dO * O) into it (LTR_DELTA_FROM_O) and no
+    attn_delta call is needed; this needs do_dq."""
     lib = _lib.load()
     _req(q, "q")
     _req(do, "dO")
@@ -153,12 +155,21 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     a.flags = ((_lib.LTR_CAUSAL if causal else 0) | (0 if do_dq else _lib.LTR_NO_DQ)
                | (0 if do_dkdv else _lib.LTR_NO_DKDV) | (_lib.LTR_DQ_BF16 if dq_direct else 0))
     a.io_dtype = _DT[q.dtype]
+    if o is not None:
+        if not do_dq:
+            raise RuntimeError("delta from o is computed by the dQ kernel: do_dq must be set")
+        if o.dtype != torch.bfloat16:
+            raise RuntimeError("delta from o needs the bf16 forward output")
+        _req(o, "o")
+        a.o, a.o_stride = o.data_ptr(), _s3(o)
+    base_flags = a.flags
     stream = _stream_ptr(q.device)
     n = len(ks)
     with torch.cuda.device(q.device):
         for start in range(0, n, _lib.LTR_MAX_CHUNKS):
             stop = min(n, start + _lib.LTR_MAX_CHUNKS)
             a.n_chunks = stop - start
+            a.flags = base_flags | (_lib.LTR_DELTA_FROM_O if (o is not None and start == 0) else 0)
             for i in range(start, stop):
                 ch = a.chunk[i - start]
                 ch.k, ch.v = ks[i].data_ptr(), vs[i].data_ptr()
@@ -210,14 +221,16 @@ class BlockAttentionFunction(torch.autograd.Function):
         if do.stride(3) != 1:
             do = do.contiguous()
         do = do.to(q.dtype)
-        delta = attn_delta(o, do)
+        fuse = o.dtype == torch.bfloat16            # DELTA computed by the dQ kernel from o
+        delta = (torch.empty(lse.shape, dtype=torch.float32, device=q.device) if fuse else attn_delta(o, do))
         # one launch sees every chunk: dQ is written as bf16 by the kernel; otherwise it accumulates in fp32
         direct = n_chunks <= _lib.LTR_MAX_CHUNKS
         dq_acc = (torch.empty(q.shape, dtype=torch.bfloat16, device=q.device) if direct
                   else torch.zeros(q.shape, dtype=torch.float32, device=q.device))
         dk_accs = [torch.zeros(k.shape, dtype=torch.float32, device=q.device) for k in ks]
         dv_accs = [torch.zeros(v.shape, dtype=torch.float32, device=q.device) for v in vs]
-        attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale)
+        attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale,
+                            o=o if fuse else None)
         dq = dq_acc if direct else cast_to_bf16(dq_acc)
         dks = [cast_to_bf16(x) for x in dk_accs]
         dvs = [cast_to_bf16(x) for x in dv_accs]

@@ -75,7 +75,9 @@ struct BwdParams {
     const void *q;
     const void *d_o;
     const float *lse;
-    const float *delta;
+    float *delta;      // read; written by the dQ kernel with LTR_DELTA_FROM_O
+    const void *o;     // bf16 forward output, read with LTR_DELTA_FROM_O only
+    long long os_[3];
     void *dq;          // fp32 accumulator, or bf16 result with LTR_DQ_BF16
     int B, Hq, Hkv, n_rep;
     int Sq, n_qtiles;
@@ -1177,9 +1179,22 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
             qreg[kb] = as_bf16x8(*(const uint4 *)(qp + kb * 16 + 8 * hh));
             doreg[kb] = as_bf16x8(*(const uint4 *)(dop + kb * 16 + 8 * hh));
         }
+        if (p.flags & LTR_DELTA_FROM_O) {
+            // DELTA = rowsum(dO * O) of this lane's row: its half of every 16-element block, then the other half's
+            const __bf16 *op = (const __bf16 *)p.o + b * p.os_[0] + (long long)rsafe * p.os_[1] + h * p.os_[2];
+            float part = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < D / 16; kb++) {
+                const bf16x8 ov = as_bf16x8(*(const uint4 *)(op + kb * 16 + 8 * hh));
+#pragma unroll
+                for (int e = 0; e < 8; e++) part += (float)ov[e] * (float)doreg[kb][e];
+            }
+            dlt = xhalf_sum(part);
+            if (row_ok && hh == 0) p.delta[((long long)b * p.Hq + h) * p.Sq + my_row] = dlt;
+        }
         if (row_ok) {
             lse2 = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row] * LTR_LOG2E;
-            dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
+            if (!(p.flags & LTR_DELTA_FROM_O)) dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
         }
     }
     f32x16 zero16;
@@ -1491,7 +1506,9 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16)) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O)) return LTR_EINVAL;
+    const bool fused_delta = a->flags & LTR_DELTA_FROM_O;
+    if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
@@ -1503,6 +1520,8 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     for (int i = 0; i < 3; i++)
         if (a->dq_stride[i] < 0) return LTR_EINVAL;
     if (do_dq && !strides_ok(a->dq_stride, (a->flags & LTR_DQ_BF16) ? 2 : 4)) return LTR_EALIGN;
+    if (fused_delta && (!aligned16(a->o) || !strides_ok(a->o_stride, 2))) return LTR_EALIGN;
+    if (fused_delta && (a->Sq + 64) * a->o_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     if ((a->Sq + 63) / 64 > BwdLds<128>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
     if ((a->Sq + 64) * a->q_stride[1] >= 0x7fffffffLL || (a->Sq + 64) * a->do_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     BwdParams p;
@@ -1528,6 +1547,8 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     p.d_o = a->d_o;
     p.lse = a->lse;
     p.delta = a->delta;
+    p.o = a->o;
+    for (int i = 0; i < 3; i++) p.os_[i] = fused_delta ? a->o_stride[i] : 0;
     p.dq = a->dq;
     p.B = a->B;
     p.Hq = a->Hq;
@@ -1558,12 +1579,13 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (rc) return rc;
     const long long nblk_q = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
     if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
+    // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
     if (a->D == 128) {
-        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
         if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
+        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
     } else {
-        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
         if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
+        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }

@@ -369,5 +369,19 @@ def test_dq_written_as_bf16_equals_accumulate_then_cast(ltr):
     direct = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device="cuda")
     ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, direct, dks, dvs, 0, None, True, do_dkdv=False)
     assert torch.equal(direct, ltr.cast_to_bf16(acc))
+    # LTR_DELTA_FROM_O: the dQ kernel computes DELTA from o and leaves it in the workspace for the dK/dV kernel
+    ws = torch.full(delta.shape, float("nan"), dtype=torch.float32, device="cuda")
+    direct2 = torch.empty_like(direct)
+    ltr.attn_bwd_accumulate(q, do, lse, ws, ks, vs, pos0, direct2, dks, dvs, 0, None, True, o=o)
+    assert (ws - delta).abs().max().item() < 1e-4 * delta.abs().max().item() + 1e-5
+    assert (direct2.float() - direct.float()).abs().max().item() < 2e-2 * direct.float().abs().max().item()
+    dk_sep = torch.zeros_like(dkf)
+    dv_sep = torch.zeros_like(dvf)
+    ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, acc, [dk_sep[:, :200], dk_sep[:, 200:]],
+                            [dv_sep[:, :200], dv_sep[:, 200:]], 0, None, True, do_dq=False)
+    assert (dkf - dk_sep).abs().max().item() < 1e-3 * dk_sep.abs().max().item()
+    assert (dvf - dv_sep).abs().max().item() < 1e-3 * dv_sep.abs().max().item()
+    with pytest.raises(RuntimeError):
+        ltr.attn_bwd_accumulate(q, do, lse, ws, ks, vs, pos0, direct2, dks, dvs, 0, None, True, do_dq=False, o=o)
     with pytest.raises(RuntimeError):
         ltr.attn_bwd_accumulate(q, do, lse, delta, ks * 20, vs * 20, pos0 * 20, direct, dks * 20, dvs * 20, 0, None, True)

@@ -28,7 +28,7 @@ def test_header_symbols_exported():
     assert declared == set(L.EXPORTS), declared
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.ltr_abi_version() == 1
+    assert lib.ltr_abi_version() == 2
     assert lib.ltr_strerror(0) == b"ok" and b"aligned" in lib.ltr_strerror(-3)
 
 
@@ -38,7 +38,7 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(L.KvChunk) == 48
     assert ctypes.sizeof(L.FwdArgs) == 3 * 8 + 4 * 4 + 8 + 4 * 24 + 16 + 8 + 4 * 5 + 4 + 32 * 48
     assert ctypes.sizeof(L.DeltaArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
-    assert ctypes.sizeof(L.BwdArgs) == 5 * 8 + 4 * 4 + 8 + 7 * 24 + 16 + 8 + 4 * 4 + 32 * 48
+    assert ctypes.sizeof(L.BwdArgs) == 5 * 8 + 4 * 4 + 8 + 7 * 24 + 16 + 8 + 4 * 4 + 32 * 48 + 8 + 24
     assert ctypes.sizeof(L.RopeArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
 
 
