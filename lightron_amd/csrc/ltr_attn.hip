@@ -388,15 +388,16 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     f32x16 oacc[D / 32];
 #pragma unroll
     for (int i = 0; i < D / 32; i++) oacc[i] = zero16;
-    // Online softmax state of this lane's query row.  mc is the reference point of the exponent; it
-    // follows the running max lazily: it moves only when some row of the wave would otherwise exceed
-    // exp2(LAZY) (P keeps its relative precision, l is accumulated in fp32 and LSE = mc*ln2 + log(l)
-    // is unaffected), so the rescale of the O
-    // accumulator is a rare wave-uniform branch instead of 64 multiplies per tile.
-    float mc = -INFINITY;     // reference point in the exp2 domain: m * scale * log2(e); -inf before the first key
+    // Online softmax state of this lane's query row.  mc is the reference point of the exponent (exp2 domain:
+    // m * scale * log2(e)).  It does not follow the running max: P = exp2(s*c2 - mc) keeps its relative precision
+    // whatever mc is, l and O accumulate in fp32 and LSE = mc*ln2 + log(l) is unaffected, so mc only has to keep
+    // the row sum inside [TINY, BIG] where neither overflow nor flushed small terms matter.  That is checked on
+    // the row sum of each tile (two compares), and the row max is only computed on the rare tile that fails the
+    // check: the common tile has no max reduction and no rescale of the O accumulator.
+    float mc = 0.f;
     float l_run = 0.f;        // this lane's partial row sum (its 32 of the 64 keys per tile)
     const float c2 = p.scale * LTR_LOG2E;
-    constexpr float LAZY = 8.f;
+    constexpr float BIG = 1.152921504606846976e18f, TINY = 8.673617379884035472e-19f;   // 2^60, 2^-60
 
     // tile iterator over (chunk, key tile)
     // The fields of the chunk being loaded live in scalar registers and are re-read from the argument
@@ -487,23 +488,48 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
                     s[nb][r] = vis ? s[nb][r] : -INFINITY;
                 }
         }
-        // t = s*c2 - reference (exp2 domain); the max is taken over t so the common case (reference stays)
-        // needs no second pass, and an arithmetic result needs no NaN canonicalisation before v_max3
-        const float mc_eff = (mc == -INFINITY) ? 0.f : mc;
+        // t = s*c2 - reference (exp2 domain), P = exp2(t) rounded to bf16, row sum of the rounded P (what PV uses)
 #pragma unroll
         for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[nb][r] = s[nb][r] * c2 - mc_eff;
-        float mx = fmaxf(s[0][0], s[1][0]);
+            for (int r = 0; r < 16; r++) s[nb][r] = s[nb][r] * c2 - mc;
+        PackedTile pt[2];
+        bf16x2 ones;
+        ones[0] = (__bf16)1.0f;
+        ones[1] = (__bf16)1.0f;
+        float l_tile = 0.f;
+        auto exponentials = [&]() {
+            l_tile = 0.f;
 #pragma unroll
-        for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
-        mx = xhalf_max(mx);
-        const bool grow = (mc == -INFINITY) ? (mx > -INFINITY) : (mx > LAZY);
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-            const float mc_new = fmaxf(mc, mc_eff + mx);          // stays -inf while the row has seen no key
-            const float mc_new_eff = (mc_new == -INFINITY) ? 0.f : mc_new;
-            const float alpha = (mc_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mc - mc_new);
-            const float shift = mc_new_eff - mc_eff;
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    bf16x2 pr;
+                    pr[0] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j]);
+                    pr[1] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j + 1]);
+                    l_tile = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_tile, false);
+                    pt[nb].u[j] = __builtin_bit_cast(unsigned, pr);
+                }
+        };
+        exponentials();
+        // in range: the tile's sum did not overflow and the row has a healthy sum by now (a lane sees half of the
+        // row's keys, so its partial sum can lag behind the row's: that only costs a visit of the branch below)
+        const bool out_of_range = !(l_tile < BIG) || !(l_run + l_tile >= TINY);
+        if (__builtin_amdgcn_ballot_w64(out_of_range) != 0) {
+            float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+            mx = xhalf_max(mx);                       // row max of t over the tile (-inf: no visible key)
+            const float l_row = xhalf_sum(l_run), lt_row = xhalf_sum(l_tile);   // whole-row sums: both halves agree
+            const bool row_bad = !(lt_row < BIG) || !(l_row + lt_row >= TINY);
+            // New reference for a row that is out of range: the larger of the tile's max and the magnitude of the
+            // history (log2 of its sum), so that neither overflows after the move; with a history never below -126, so
+            // that the factor applied to it stays finite.  Rows that are in range, and rows that have seen no key at
+            // all, keep theirs.
+            const float hist = l_row > 0.f ? __log2f(l_row) : -INFINITY;
+            const float target = fmaxf(mx, hist);
+            const float shift = (row_bad && target > -INFINITY) ? (l_row > 0.f ? fmaxf(target, -126.f) : target) : 0.f;
+            const float alpha = l_row > 0.f ? __builtin_amdgcn_exp2f(-shift) : 1.f;
             l_run *= alpha;
 #pragma unroll
             for (int i = 0; i < D / 32; i++)
@@ -513,22 +539,10 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             for (int nb = 0; nb < 2; nb++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) s[nb][r] -= shift;
-            mc = mc_new;
+            mc += shift;
+            exponentials();
         }
-        PackedTile pt[2];
-        bf16x2 ones;
-        ones[0] = (__bf16)1.0f;
-        ones[1] = (__bf16)1.0f;
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                bf16x2 pr;
-                pr[0] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j]);
-                pr[1] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j + 1]);
-                l_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_run, false);   // sums the rounded P that PV uses
-                pt[nb].u[j] = __builtin_bit_cast(unsigned, pr);
-            }
+        l_run += l_tile;
         __builtin_amdgcn_s_setprio(1);
         {
             const bf16x8 pb[4] = {operand_of(pt[0], 0), operand_of(pt[0], 1), operand_of(pt[1], 0), operand_of(pt[1], 1)};

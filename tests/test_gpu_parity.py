@@ -385,3 +385,40 @@ def test_dq_written_as_bf16_equals_accumulate_then_cast(ltr):
         ltr.attn_bwd_accumulate(q, do, lse, ws, ks, vs, pos0, direct2, dks, dvs, 0, None, True, do_dq=False, o=o)
     with pytest.raises(RuntimeError):
         ltr.attn_bwd_accumulate(q, do, lse, delta, ks * 20, vs * 20, pos0 * 20, direct, dks * 20, dvs * 20, 0, None, True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["huge_positive", "huge_negative", "mixed_rows", "growing"])
+def test_extreme_logits(ltr, case):
+    """Scores far outside the range where exp2 of (score - fixed reference) is representable: the forward's
+    range check on the row sums must move the reference (up on overflow, down when everything would flush) and
+    still match the dense fp64 formula; causal, two KV chunks, GQA."""
+    g = torch.Generator().manual_seed(13)
+    B, S, Hq, Hkv, D = 1, 256, 4, 2, 64
+    q = torch.randn(B, S, Hq, D, generator=g)
+    k = torch.randn(B, S, Hkv, D, generator=g)
+    v = torch.randn(B, S, Hkv, D, generator=g)
+    u = torch.randn(D, generator=g)
+    u = u / u.norm()
+    if case == "huge_positive":        # scores ~ +40^2 / 8 = +200 natural units = +290 in the exp2 domain
+        q, k = q + 40 * u, k + 40 * u
+    elif case == "huge_negative":      # every score ~ -200: exp2(score) flushes to zero with the initial reference
+        q, k = q + 40 * u, k - 40 * u
+    elif case == "mixed_rows":         # some rows huge positive, some huge negative, some ordinary
+        q[:, 0::3] += 40 * u
+        q[:, 1::3] -= 40 * u
+        k = k + 40 * u
+    else:                              # the row max grows from chunk to chunk by hundreds
+        k[:, S // 2:] += 60 * u
+        q = q + 20 * u
+    q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
+    pos = torch.arange(S)
+    o_ref, lse_ref = orc.dense_attention(q.float(), k.float(), v.float(), pos, pos, True)
+    ks, vs = [k[:, :128].cuda(), k[:, 128:].cuda()], [v[:, :128].cuda(), v[:, 128:].cuda()]
+    for stepwise in (False, True):
+        qd = q.cuda().requires_grad_(True)
+        o, lse = ltr.block_attention(qd, ks, vs, [0, 128], 0, None, causal=True, stepwise=stepwise)
+        assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+        assert (o.float().cpu() - o_ref).abs().max() < 3e-2
+        # LSE comes from sums of bf16-rounded P: 1e-2 absolute as elsewhere for bf16, plus 1e-3 of its size
+        assert ((lse.cpu() - lse_ref).abs() <= 1e-2 + 1e-3 * lse_ref.abs()).all()
