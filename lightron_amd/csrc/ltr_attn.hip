@@ -4,8 +4,8 @@
 // Kernel map
 //   fwd_bf16_kernel<D>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a block of
 //                        8 waves owns 256 query rows, a wave 32 of them, so a lane owns ONE query:
-//                        the row max / sum are
-//                        in-lane reductions plus one v_permlane32_swap, and P^T leaves the
+//                        the row sums are in-lane reductions (no running max: the reference of the
+//                        exponent moves only when a row sum leaves its safe range), and P^T leaves the
 //                        first GEMM already in the B-operand layout of the second.  64-key K
 //                        and V tiles go global -> LDS directly (no staging registers) into
 //                        unpadded, XOR-swizzled, double-buffered tiles, one barrier per tile;
