@@ -1281,6 +1281,16 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
             __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
             lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, sw, Vs + (nb * 32 + l32) * D, sw, qreg, doreg, s, dp);
             __builtin_amdgcn_s_setprio(0);
+            // mask fix-up (tail of the chunk, diagonal tiles, rows past the end): wave-uniform branch touching S only;
+            // an invisible entry gets S = -inf, so P = 0 and dS = 0
+            if (need_mask) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                    const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
+                    s[r] = vis ? s[r] : -INFINITY;
+                }
+            }
             PackedTile ds;
 #pragma unroll
             for (int j = 0; j < 8; j++) {
@@ -1290,15 +1300,6 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
                     const int r = 2 * j + e;
                     const float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2);
                     dsv[e] = pv * (dp[r] - dlt);
-                }
-                if (need_mask) {
-#pragma unroll
-                    for (int e = 0; e < 2; e++) {
-                        const int r = 2 * j + e;
-                        const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
-                        const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
-                        dsv[e] = vis ? dsv[e] : 0.f;
-                    }
                 }
                 ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
             }
