@@ -38,13 +38,22 @@ def _same_strides(ts: Sequence[torch.Tensor]) -> bool:
     return all(t.stride() == s0 for t in ts)
 
 
+def _common_layout(ts):
+    """Chunks whose strides differ (separate tensors of unequal length have different batch strides) are
+    packed once into one [B, sum S, H, D] buffer and returned as its sequence slices, which share one triple."""
+    if _same_strides(ts):
+        return list(ts)
+    buf = torch.cat([t for t in ts], dim=1)
+    out, start = [], 0
+    for t in ts:
+        out.append(buf[:, start:start + t.shape[1]])
+        start += t.shape[1]
+    return out
+
+
 def _norm_chunks(ks, vs):
     """The ABI carries one stride triple for all K chunks and one for all V chunks."""
-    if not _same_strides(ks):
-        ks = [k.contiguous() for k in ks]
-    if not _same_strides(vs):
-        vs = [v.contiguous() for v in vs]
-    return list(ks), list(vs)
+    return _common_layout(ks), _common_layout(vs)
 
 
 def _qpos(q_pos0, Sq, q_split):
@@ -227,13 +236,20 @@ class BlockAttentionFunction(torch.autograd.Function):
         direct = n_chunks <= _lib.LTR_MAX_CHUNKS
         dq_acc = (torch.empty(q.shape, dtype=torch.bfloat16, device=q.device) if direct
                   else torch.zeros(q.shape, dtype=torch.float32, device=q.device))
-        dk_accs = [torch.zeros(k.shape, dtype=torch.float32, device=q.device) for k in ks]
-        dv_accs = [torch.zeros(v.shape, dtype=torch.float32, device=q.device) for v in vs]
+        # one fp32 buffer per gradient, sliced along the sequence: every chunk's accumulator has the same strides
+        lens = [k.shape[1] for k in ks]
+        shape = (ks[0].shape[0], sum(lens), ks[0].shape[2], ks[0].shape[3])
+        dk_buf = torch.zeros(shape, dtype=torch.float32, device=q.device)
+        dv_buf = torch.zeros(shape, dtype=torch.float32, device=q.device)
+        offs = [sum(lens[:i]) for i in range(len(lens))]
+        dk_accs = [dk_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+        dv_accs = [dv_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale,
                             o=o if fuse else None)
         dq = dq_acc if direct else cast_to_bf16(dq_acc)
-        dks = [cast_to_bf16(x) for x in dk_accs]
-        dvs = [cast_to_bf16(x) for x in dv_accs]
+        dk16, dv16 = cast_to_bf16(dk_buf), cast_to_bf16(dv_buf)
+        dks = [dk16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+        dvs = [dv16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         return (dq, None, None, None, None, None, None, None, None, *dks, *dvs)
 
 

@@ -1207,7 +1207,10 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
             if (row_ok && hh == 0) p.delta[((long long)b * p.Hq + h) * p.Sq + my_row] = dlt;
         }
         if (row_ok) {
-            lse2 = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row] * LTR_LOG2E;
+            // a row that saw no key has LSE = -inf: give it +inf like a row past the end, so that P = exp2(-inf) = 0
+            // whatever S is (S = -inf after the mask fix-up would otherwise meet -(-inf))
+            const float lse_row = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row];
+            lse2 = lse_row == -INFINITY ? INFINITY : lse_row * LTR_LOG2E;
             if (!(p.flags & LTR_DELTA_FROM_O)) dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
         }
     }

@@ -422,3 +422,61 @@ def test_extreme_logits(ltr, case):
         assert (o.float().cpu() - o_ref).abs().max() < 3e-2
         # LSE comes from sums of bf16-rounded P: 1e-2 absolute as elsewhere for bf16, plus 1e-3 of its size
         assert ((lse.cpu() - lse_ref).abs() <= 1e-2 + 1e-3 * lse_ref.abs()).all()
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_shapes_sweep(ltr, seed):
+    """Seeded sweep over shapes the fixed cases do not hit: ragged Sq across the 256-row block size, 1-4 KV chunks
+    of unequal length (slices of one buffer), arbitrary chunk positions, a two-segment query (q_split) or not,
+    causal or not, GQA ratios, both head dims; forward and all gradients against the dense oracle with
+    explicit positions."""
+    import random
+    rnd = random.Random(1000 + seed)
+    g = torch.Generator().manual_seed(2000 + seed)
+    D = rnd.choice([64, 128])
+    Hkv = rnd.choice([1, 2])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    B = rnd.choice([1, 2])
+    Sq = rnd.choice([1, 31, 64, 200, 255, 256, 257, 300, 513, 640])
+    n_ch = rnd.randint(1, 4)
+    sks = [rnd.choice([1, 17, 64, 100, 128, 191, 256, 330]) for _ in range(n_ch)]
+    causal = rnd.random() < 0.7
+    # chunk positions: disjoint ranges in random order; query segments placed among them
+    starts, p = [], rnd.randint(0, 50)
+    for sk in sks:
+        starts.append(p)
+        p += sk + rnd.randint(0, 40)
+    order = list(range(n_ch))
+    rnd.shuffle(order)
+    q_split = rnd.choice([None, rnd.randint(1, Sq)]) if Sq > 1 else None
+    if q_split is None or q_split == Sq:
+        q_split, qp = None, rnd.randint(0, p)
+        q_pos = torch.arange(qp, qp + Sq)
+        q_pos0 = qp
+    else:
+        a0, a1 = rnd.randint(0, p), rnd.randint(0, p + 200)
+        q_pos = torch.cat([torch.arange(a0, a0 + q_split), torch.arange(a1, a1 + Sq - q_split)])
+        q_pos0 = (a0, a1)
+    q = _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    do = _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    kbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
+    vbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
+    offs = [sum(sks[:i]) for i in range(n_ch)]
+    k_pos = torch.cat([torch.arange(starts[i], starts[i] + sks[i]) for i in range(n_ch)])
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), kbuf.float(), vbuf.float(), do.float(),
+                                                                         q_pos, k_pos, causal)
+    kd, vd = kbuf.cuda().requires_grad_(True), vbuf.cuda().requires_grad_(True)
+    qd = q.cuda().requires_grad_(True)
+    ks = [kd[:, offs[i]:offs[i] + sks[i]] for i in order]
+    vs = [vd[:, offs[i]:offs[i] + sks[i]] for i in order]
+    o, lse = ltr.block_attention(qd, ks, vs, [starts[i] for i in order], q_pos0, q_split, causal=causal)
+    o.backward(do.cuda())
+    seen = torch.isfinite(lse_ref)                       # rows that see at least one key
+    assert torch.equal(torch.isfinite(lse.cpu()), seen)
+    assert (o.float().cpu() - o_ref.float()).abs().max() < O_TOL_BF16
+    assert (lse.cpu()[seen] - lse_ref.float()[seen]).abs().max() < LSE_TOL_BF16 if seen.any() else True
+    for got, ref in ((qd.grad, dq_ref), (kd.grad, dk_ref), (vd.grad, dv_ref)):
+        if ref.abs().max() > 0:
+            assert _rel(got.cpu(), ref) < GRAD_RTOL_BF16
+        else:
+            assert got.abs().max() == 0
