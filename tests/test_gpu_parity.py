@@ -424,7 +424,7 @@ def test_extreme_logits(ltr, case):
         assert ((lse.cpu() - lse_ref).abs() <= 1e-2 + 1e-3 * lse_ref.abs()).all()
 
 
-@pytest.mark.parametrize("seed", list(range(12)))
+@pytest.mark.parametrize("seed", list(range(24)))
 def test_random_shapes_sweep(ltr, seed):
     """Seeded sweep over shapes the fixed cases do not hit: ragged Sq across the 256-row block size, 1-4 KV chunks
     of unequal length (slices of one buffer), arbitrary chunk positions, a two-segment query (q_split) or not,
@@ -478,5 +478,47 @@ def test_random_shapes_sweep(ltr, seed):
     for got, ref in ((qd.grad, dq_ref), (kd.grad, dk_ref), (vd.grad, dv_ref)):
         if ref.abs().max() > 0:
             assert _rel(got.cpu(), ref) < GRAD_RTOL_BF16
-        else:
-            assert got.abs().max() == 0
+        else:   # e.g. one visible key per row: the exact gradient is 0, the kernels leave rounding noise
+            assert got.abs().max() < 1e-3
+
+
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_random_shapes_sweep_fp32_and_stepwise(ltr, seed):
+    """The same kind of sweep for the fp32 forward kernel and for the step-wise path (one launch per KV chunk, the
+    (O, LSE) merge in the epilogue), forward only; fp32 inputs to 1e-4, bf16 inputs to the bf16 tolerances."""
+    import random
+    rnd = random.Random(5000 + seed)
+    g = torch.Generator().manual_seed(6000 + seed)
+    dtype = rnd.choice([torch.float32, torch.bfloat16])
+    D = rnd.choice([64, 128])
+    Hkv = rnd.choice([1, 2])
+    Hq = Hkv * rnd.choice([1, 2])
+    B = rnd.choice([1, 2])
+    Sq = rnd.choice([1, 63, 64, 65, 130, 256, 300])
+    n_ch = rnd.randint(1, 4)
+    sks = [rnd.choice([1, 17, 64, 100, 128, 191]) for _ in range(n_ch)]
+    causal = rnd.random() < 0.7
+    starts, p = [], rnd.randint(0, 30)
+    for sk in sks:
+        starts.append(p)
+        p += sk
+    qp = rnd.randint(0, p)
+    q_pos = torch.arange(qp, qp + Sq)
+    q = _randn((B, Sq, Hq, D), g, dtype)
+    kbuf = _randn((B, sum(sks), Hkv, D), g, dtype)
+    vbuf = _randn((B, sum(sks), Hkv, D), g, dtype)
+    offs = [sum(sks[:i]) for i in range(n_ch)]
+    k_pos = torch.cat([torch.arange(starts[i], starts[i] + sks[i]) for i in range(n_ch)])
+    o_ref, lse_ref = orc.dense_attention(q.float(), kbuf.float(), vbuf.float(), q_pos, k_pos, causal)
+    kd, vd = kbuf.cuda(), vbuf.cuda()
+    ks = [kd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    vs = [vd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    o_tol, l_tol = (F32_TOL, F32_TOL) if dtype == torch.float32 else (O_TOL_BF16, LSE_TOL_BF16)
+    seen = torch.isfinite(lse_ref)
+    for stepwise in (False, True):
+        with torch.no_grad():
+            o, lse = ltr.block_attention(q.cuda(), ks, vs, starts, qp, None, causal=causal, stepwise=stepwise)
+        assert torch.equal(torch.isfinite(lse.cpu()), seen)
+        assert (o.float().cpu() - o_ref.float()).abs().max() < o_tol
+        if seen.any():
+            assert (lse.cpu()[seen] - lse_ref.float()[seen]).abs().max() < l_tol
