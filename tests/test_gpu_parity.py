@@ -522,3 +522,63 @@ def test_random_shapes_sweep_fp32_and_stepwise(ltr, seed):
         assert (o.float().cpu() - o_ref.float()).abs().max() < o_tol
         if seen.any():
             assert (lse.cpu()[seen] - lse_ref.float()[seen]).abs().max() < l_tol
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_ring_sweep_all_ranks_forward_backward(ltr, seed):
+    """ring_attention_kernel with a LocalRing for every rank of a random ring (world size, layout, causal or not,
+    GQA, step-wise or fused): the ranks' outputs, gathered back to sequence order, against dense attention on the
+    whole sequence; dQ per rank and dK/dV summed over the ranks against its gradients."""
+    import random
+    rnd = random.Random(7000 + seed)
+    g = torch.Generator().manual_seed(8000 + seed)
+    W = rnd.choice([1, 2, 3, 4, 5])
+    layout = rnd.choice(["contiguous", "zigzag"])
+    causal = rnd.random() < 0.7
+    stepwise = rnd.random() < 0.4
+    D = rnd.choice([64, 128])
+    Hkv = rnd.choice([1, 2])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    B = rnd.choice([1, 2])
+    Sl = rnd.choice([2, 34, 64, 96, 130, 256])
+    S = W * Sl
+    q, do = (_randn((B, S, Hq, D), g, torch.bfloat16) for _ in range(2))
+    k, v = (_randn((B, S, Hkv, D), g, torch.bfloat16) for _ in range(2))
+    pos = torch.arange(S)
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), k.float(), v.float(), do.float(), pos, pos, causal)
+    share = [orc.zigzag_positions(r, W, S) if layout == "zigzag" else orc.contiguous_positions(r, Sl) for r in range(W)]
+    kd = [k[:, share[r]].contiguous().cuda().requires_grad_(True) for r in range(W)]
+    vd = [v[:, share[r]].contiguous().cuda().requires_grad_(True) for r in range(W)]
+    for r in range(W):
+        qr = q[:, share[r]].contiguous().cuda().requires_grad_(True)
+        ring = ltr.LocalRing(r, W, kv=list(zip(kd, vd)), causal=causal, layout=layout, stepwise=stepwise)
+        o = ltr.ring_attention_kernel(qr, kd[r], vd[r], ring, None)
+        o.backward(do[:, share[r]].contiguous().cuda())
+        assert (o.float().cpu() - o_ref[:, share[r]].float()).abs().max() < O_TOL_BF16
+        assert (ring.last_lse.cpu() - lse_ref[:, :, share[r]].float()).abs().max() < LSE_TOL_BF16
+        assert _rel(qr.grad.cpu(), dq_ref[:, share[r]]) < GRAD_RTOL_BF16
+    # each rank's backward added a bf16-rounded contribution to the chunks' .grad: W roundings instead of one
+    dk = torch.zeros_like(dk_ref)
+    dv = torch.zeros_like(dv_ref)
+    for r in range(W):
+        dk[:, share[r]] = kd[r].grad.cpu().double()
+        dv[:, share[r]] = vd[r].grad.cpu().double()
+    assert _rel(dk, dk_ref) < GRAD_RTOL_BF16 and _rel(dv, dv_ref) < GRAD_RTOL_BF16
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_rope_sweep_bit_exact(ltr, seed):
+    """ltr_rope_apply on random shapes, dtypes, layouts and starting positions against the oracle, bit for bit."""
+    import random
+    rnd = random.Random(9000 + seed)
+    g = torch.Generator().manual_seed(9100 + seed)
+    dtype = rnd.choice([torch.float32, torch.bfloat16])
+    B, S, H = rnd.choice([1, 2, 3]), rnd.choice([1, 7, 64, 129]), rnd.choice([1, 2, 5])
+    D = rnd.choice([8, 16, 64, 96, 128])
+    p0 = rnd.choice([0, 5, 1000, 100000])
+    x = _randn((B, H, S, D), g, dtype) if rnd.random() < 0.5 else _randn((B, S, H, D), g, dtype).transpose(1, 2)
+    xv = x.transpose(1, 2)                                    # [B, S, H, D] view, one of the two memory layouts
+    fc = orc.precompute_freqs_cis(D, p0 + S)[p0:]
+    ref, _ = orc.apply_rotary_emb(xv, xv, fc)
+    got, _ = ltr.apply_rotary_emb(xv.cuda(), xv.cuda(), fc.cuda())
+    assert got.dtype == dtype and torch.equal(got.cpu(), ref)
