@@ -210,11 +210,12 @@ def test_cast_kernel(ltr):
     assert torch.equal(ltr.cast_to_bf16(x), x.to(torch.bfloat16))
 
 
-def test_ulysses_module_matches_oracle(ltr):
-    """Config 5's layout at reduced size: 4 ranks, sequence shards [B, S/4, H, D] -> head shards,
-    attention, and back; literal (exchange-by-exchange) and zero-copy paths vs the oracle."""
+@pytest.mark.parametrize("W,B,Sl,H,D", [(4, 2, 64, 8, 64), (2, 1, 50, 2, 128), (3, 1, 40, 6, 64), (8, 1, 32, 8, 64)])
+def test_ulysses_module_matches_oracle(ltr, W, B, Sl, H, D):
+    """Config 5's layout at reduced size (and other ring sizes / ragged shard lengths): W ranks, sequence shards
+    [B, S/W, H, D] -> head shards, attention, and back; literal (exchange-by-exchange) and zero-copy paths vs the
+    oracle."""
     import torch.nn as nn
-    W, B, Sl, H, D = 4, 2, 64, 8, 64
     dim = H * D
 
     class Attn(nn.Module):
