@@ -231,25 +231,35 @@ def test_ulysses_module_matches_oracle(ltr, W, B, Sl, H, D):
     attn = Attn().to(torch.bfloat16)
     x = ((torch.rand(W, B, Sl, dim) * 2 - 1) * 0.5).to(torch.bfloat16)
     fc = orc.precompute_freqs_cis(D, W * Sl)
-    # oracle: projections in fp32 torch on the CPU, exchange, RoPE, dense causal attention, exchange back
-    with torch.no_grad():
-        xq, xk, xv = (lin(x).view(W, B, Sl, H, D) for lin in (attn.wq, attn.wk, attn.wv))
-        sq, sk, sv = (orc.seq_all_to_all([t[r] for r in range(W)], 2, 1) for t in (xq, xk, xv))
-        outs = []
-        pos = torch.arange(W * Sl)
-        for r in range(W):
-            rq, rk = orc.apply_rotary_emb(sq[r], sk[r], fc)
-            o, _ = orc.dense_attention(rq, rk, sv[r], pos, pos, True)
-            outs.append(o.to(torch.bfloat16))
-        back = orc.seq_all_to_all(outs, 1, 2)
-        ref = torch.stack([attn.wo(b.flatten(2)) for b in back], 0)
+    # oracle: projections in fp32 torch on the CPU, exchange, RoPE, dense causal attention, exchange back; with
+    # autograd, so that the gradients of the input and of the four weights are checked as well
+    dy = ((torch.rand(W, B, Sl, dim) * 2 - 1) * 0.1).to(torch.bfloat16)
+    ws = {n: p_.detach().float().requires_grad_(True) for n, p_ in attn.named_parameters()}
+    xr = x.float().requires_grad_(True)
+    xq, xk, xv = ((xr @ ws[n].T).view(W, B, Sl, H, D) for n in ("wq.weight", "wk.weight", "wv.weight"))
+    sq, sk, sv = (orc.seq_all_to_all([t[r] for r in range(W)], 2, 1) for t in (xq, xk, xv))
+    outs = []
+    pos = torch.arange(W * Sl)
+    for r in range(W):
+        rq, rk = orc.apply_rotary_emb(sq[r], sk[r], fc)
+        o, _ = orc.dense_attention(rq, rk, sv[r], pos, pos, True)
+        outs.append(o.float())
+    back = orc.seq_all_to_all(outs, 1, 2)
+    ref = torch.stack([b_.flatten(2) @ ws["wo.weight"].T for b_ in back], 0)
+    ref.backward(dy.float())
     attn_d = attn.cuda()
+    rel = lambda a, b_: ((a.float().cpu() - b_).norm() / b_.norm()).item()
     for literal in (True, False):
         mod = ltr.ContextParallelAttention(attn_d, Args, cp_group=ltr.LocalCPGroup(W), literal=literal)
-        with torch.no_grad():
-            y = mod(x.cuda(), fc.cuda())
+        attn_d.zero_grad()
+        xd = x.cuda().requires_grad_(True)
+        y = mod(xd, fc.cuda())
+        y.backward(dy.cuda())
         assert y.shape == (W, B, Sl, dim)
-        assert (y.cpu().float() - ref.float()).abs().max() < 3e-2
+        assert (y.detach().cpu().float() - ref.detach()).abs().max() < 3e-2
+        assert rel(xd.grad, xr.grad) < 5e-2
+        for n, p_ in attn_d.named_parameters():
+            assert rel(p_.grad, ws[n].grad) < 5e-2, n
     # passthrough without a cp group (parallel_cp.py:161-162)
     called = {}
     attn_d.forward = lambda x_, f_: called.setdefault("y", x_)
