@@ -342,14 +342,15 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     const bool causal = p.flags & LTR_CAUSAL;
 
     // block -> (batch, kv head, q head of the group, q tile).  Consecutive block ids go to
-    // the 8 XCDs round-robin; keep all q tiles / q heads of one (batch, kv head) on one XCD
-    // so its K/V stay in that XCD's L2.  Late (heavier under a causal mask) q tiles first.
+    // the 8 XCDs round-robin; all q tiles / q heads of one (batch, kv head) run on one XCD and
+    // next to each other in time, so the blocks that are resident together stream the same K/V
+    // through that XCD's L2.  Late (heavier under a causal mask) q tiles first.
     int idx = blockIdx.x, pair, rest;
     const int P = p.B * p.Hkv;
     if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3, pp = P >> 3;
-        pair = (j % pp) * 8 + xcd;
-        rest = j / pp;
+        int xcd = idx & 7, j = idx >> 3, nr = p.n_qtiles * p.n_rep;
+        pair = (j / nr) * 8 + xcd;
+        rest = j % nr;
     } else {
         pair = idx % P;
         rest = idx / P;
@@ -830,9 +831,9 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     int idx = blockIdx.x, pair, rest;
     const int P = p.B * p.Hkv;
     if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3, pp = P >> 3;
-        pair = (j % pp) * 8 + xcd;
-        rest = j / pp;
+        int xcd = idx & 7, j = idx >> 3;
+        pair = (j / p.tiles_total) * 8 + xcd;
+        rest = j % p.tiles_total;
     } else {
         pair = idx % P;
         rest = idx / P;
@@ -1158,9 +1159,9 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     int idx = blockIdx.x, pair, rest;
     const int P = p.B * p.Hkv;
     if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3, pp = P >> 3;
-        pair = (j % pp) * 8 + xcd;
-        rest = j / pp;
+        int xcd = idx & 7, j = idx >> 3, nr = ((p.Sq + BM - 1) / BM) * p.n_rep;
+        pair = (j / nr) * 8 + xcd;
+        rest = j % nr;
     } else {
         pair = idx % P;
         rest = idx / P;
