@@ -325,10 +325,17 @@ __device__ __forceinline__ void lds_tr_gemm(const __bf16 *T, int row0, int lane,
     }
 }
 
+// keys per K / V tile of the forward and dQ kernels
+template <int D>
+struct FwdTile {
+    static constexpr int BN = D == 64 ? 128 : 64;
+};
+
 // ------------------------------------------------------------------------------ forward, bf16
 template <int D>
 __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
-    constexpr int NW = 8, BM = 32 * NW, BN = 64;   // 8 waves (two per SIMD) share every K / V tile
+    constexpr int NW = 8, BM = 32 * NW;   // 8 waves (two per SIMD) share every K / V tile
+    constexpr int BN = FwdTile<D>::BN, NB = BN / 32;   // keys per tile: a tile moves 32 KB whatever the head dim
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
     constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
@@ -396,7 +403,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     // the row sum of each tile (two compares), and the row max is only computed on the rare tile that fails the
     // check: the common tile has no max reduction and no rescale of the O accumulator.
     float mc = 0.f;
-    float l_run = 0.f;        // this lane's partial row sum (its 32 of the 64 keys per tile)
+    float l_run = 0.f;        // this lane's partial row sum (its half of the keys of every tile)
     const float c2 = p.scale * LTR_LOG2E;
     constexpr float BIG = 1.152921504606846976e18f, TINY = 8.673617379884035472e-19f;   // 2^60, 2^-60
 
@@ -473,15 +480,20 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         // S^T of the two 32-key blocks of the tile.  The wave raises its priority while it issues MFMAs: the
         // other wave of the SIMD then fills the gaps with its softmax arithmetic instead of delaying them.
         __builtin_amdgcn_s_setprio(1);
-        f32x16 s[2] = {zero16, zero16};
-        lds_gemm_pair<D>(Ks + l32 * D, lds_swz<D>(l32) ^ hh, Ks + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, qreg, qreg,
-                         s[0], s[1]);
+        f32x16 s[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb += 2) {
+            s[nb] = zero16;
+            s[nb + 1] = zero16;
+            lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, lds_swz<D>(nb * 32 + l32) ^ hh, Ks + (nb * 32 + 32 + l32) * D,
+                             lds_swz<D>(nb * 32 + 32 + l32) ^ hh, qreg, qreg, s[nb], s[nb + 1]);
+        }
         __builtin_amdgcn_s_setprio(0);
         // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         if (need_mask) {
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++)
+            for (int nb = 0; nb < NB; nb++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
@@ -491,10 +503,10 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         }
         // t = s*c2 - reference (exp2 domain), P = exp2(t) rounded to bf16, row sum of the rounded P (what PV uses)
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++)
+        for (int nb = 0; nb < NB; nb++)
 #pragma unroll
             for (int r = 0; r < 16; r++) s[nb][r] = s[nb][r] * c2 - mc;
-        PackedTile pt[2];
+        PackedTile pt[NB];
         bf16x2 ones;
         ones[0] = (__bf16)1.0f;
         ones[1] = (__bf16)1.0f;
@@ -502,7 +514,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         auto exponentials = [&]() {
             l_tile = 0.f;
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++)
+            for (int nb = 0; nb < NB; nb++)
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     bf16x2 pr;
@@ -517,9 +529,11 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         // row's keys, so its partial sum can lag behind the row's: that only costs a visit of the branch below)
         const bool out_of_range = !(l_tile < BIG) || !(l_run + l_tile >= TINY);
         if (__builtin_amdgcn_ballot_w64(out_of_range) != 0) {
-            float mx = fmaxf(s[0][0], s[1][0]);
+            float mx = -INFINITY;
 #pragma unroll
-            for (int r = 1; r < 16; r++) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[nb][r]);
             mx = xhalf_max(mx);                       // row max of t over the tile (-inf: no visible key)
             const float l_row = xhalf_sum(l_run), lt_row = xhalf_sum(l_tile);   // whole-row sums: both halves agree
             const bool row_bad = !(lt_row < BIG) || !(l_row + lt_row >= TINY);
@@ -537,7 +551,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++)
+            for (int nb = 0; nb < NB; nb++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) s[nb][r] -= shift;
             mc += shift;
@@ -546,8 +560,10 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         l_run += l_tile;
         __builtin_amdgcn_s_setprio(1);
         {
-            const bf16x8 pb[4] = {operand_of(pt[0], 0), operand_of(pt[0], 1), operand_of(pt[1], 0), operand_of(pt[1], 1)};
-            lds_tr_gemm<D, 4>(Vs, 0, lane, pb, oacc);   // 16 keys per MFMA
+            bf16x8 pb[2 * NB];
+#pragma unroll
+            for (int kb = 0; kb < 2 * NB; kb++) pb[kb] = operand_of(pt[kb >> 1], kb & 1);
+            lds_tr_gemm<D, 2 * NB>(Vs, 0, lane, pb, oacc);   // 16 keys per MFMA
         }
         __builtin_amdgcn_s_setprio(0);
         tile_barrier();
@@ -1366,7 +1382,7 @@ int check_device() {
 
 // kernels that need more than 64 KB of dynamic LDS must opt in once per process
 template <int D>
-constexpr int fwd_lds_bytes() { return 2 * 2 * 64 * D * 2; }
+constexpr int fwd_lds_bytes() { return 2 * 2 * FwdTile<D>::BN * D * 2; }
 template <int D>
 constexpr int dq_lds_bytes() { return 2 * 2 * 64 * D * 2; }
 
