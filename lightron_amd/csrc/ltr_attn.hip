@@ -1159,7 +1159,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
 // registers as the B operand of dQ^T += K^T dS^T, whose A operand is the K tile read by transpose loads.
 template <int D>
 __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
-    constexpr int NW = 8, BM = 32 * NW, BN = 64;   // 8 waves (two per SIMD) share every K / V tile
+    constexpr int NW = 8, BM = 32 * NW, BN = FwdTile<D>::BN;   // 8 waves (two per SIMD) share every K / V tile
     constexpr int CPR = D / 8;
     constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
     constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
@@ -1292,10 +1292,10 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
         if (have_next) gload(t, par ^ 1);
 
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
-        // two 32-key halves one after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
+        // 32 keys at a time, one block after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
         // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
+        for (int nb = 0; nb < BN / 32; nb++) {
             f32x16 s = zero16, dp = zero16;
             const int sw = lds_swz<D>(nb * 32 + l32) ^ hh;       // chunk 2*kb + hh lives at (2*kb) ^ sw
             __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
@@ -1384,7 +1384,7 @@ int check_device() {
 template <int D>
 constexpr int fwd_lds_bytes() { return 2 * 2 * FwdTile<D>::BN * D * 2; }
 template <int D>
-constexpr int dq_lds_bytes() { return 2 * 2 * 64 * D * 2; }
+constexpr int dq_lds_bytes() { return 2 * 2 * FwdTile<D>::BN * D * 2; }
 
 int enable_large_lds() {
     static int done = 0;  // 0 not yet, 1 ok, -1 failed
