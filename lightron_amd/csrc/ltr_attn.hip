@@ -461,8 +461,10 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         for (int j = 0; j < 2 * NI; j++) gload_one(j, t, 0);
     }
     tile_barrier();
-    int par = 0;
-    while (have) {
+    // One tile; the loop below is unrolled over the two LDS buffers so that every LDS address is a loop-invariant
+    // per-lane register plus an immediate offset (no address arithmetic between the MFMAs).
+    auto tile_step = [&](auto par_tag) {
+        constexpr int par = decltype(par_tag)::value;
         const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
         const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + TILE;
         t++;
@@ -567,8 +569,12 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         }
         __builtin_amdgcn_s_setprio(0);
         tile_barrier();
-        par ^= 1;
         have = have_next;
+    };
+    while (have) {
+        tile_step(std::integral_constant<int, 0>{});
+        if (!have) break;
+        tile_step(std::integral_constant<int, 1>{});
     }
 
     // epilogue: normalise, optional merge with the partial result already in (o, lse)
@@ -1021,9 +1027,14 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             *(uint4 *)(slot + lane * 4) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
             *(uint4 *)(slot + 256 + lane * 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
         };
-        int buf = 0, par = 0;
+        int par = 0;
+        // In the pass over unmasked tiles both loops are unrolled over the three Q / dO buffers (buf is a compile-time
+        // constant inside a step), so that LDS addresses are loop-invariant per-lane registers plus immediate offsets;
+        // the pass over masked tiles (few steps, more live registers) keeps one loop body with buf in a register.
         if (p_role) {
-            for (bool more = true; more;) {
+            bool more = true;
+            auto p_step = [&](auto buf_tag) {
+                const int buf = buf_tag;
                 mctx.row_base = qt * BM;
                 more = advance(rep, qt);
                 const int nbuf = buf == L::NBUF - 1 ? 0 : buf + 1;
@@ -1069,18 +1080,32 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 pb[3] = operand_of(ppb, 1);
                 lds_tr_gemm<D, 2>(dOs, 32, lane, *(const bf16x8(*)[2]) & pb[2], acc);
                 __builtin_amdgcn_s_setprio(0);
-                buf = nbuf;
-                if (more) lds_store(buf);
+                if (more) lds_store(nbuf);
                 tile_barrier();
                 par ^= 1;
+            };
+            static_assert(L::NBUF == 3, "unrolled over three buffers");
+            if (MASK) {
+                for (int buf = 0; more; buf = buf == L::NBUF - 1 ? 0 : buf + 1) p_step(buf);
+            } else {
+                for (;;) {
+                    p_step(std::integral_constant<int, 0>{});
+                    if (!more) break;
+                    p_step(std::integral_constant<int, 1>{});
+                    if (!more) break;
+                    p_step(std::integral_constant<int, 2>{});
+                    if (!more) break;
+                }
             }
             tile_barrier();                        // step T: only the dS waves have work
         } else {
             bool more = advance(rep, qt);          // step 0: staging duties only
             if (more) gload(rep, qt, 1);
             tile_barrier();
-            for (;;) {
-                const bool had_next = more;
+            bool had_next = true;
+            auto ds_step = [&](auto buf_tag) {
+                const int buf = buf_tag;
+                had_next = more;
                 if (more) {
                     more = advance(rep, qt);
                     if (more) gload(rep, qt, buf + 2 >= L::NBUF ? buf + 2 - L::NBUF : buf + 2);
@@ -1127,9 +1152,19 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 lds_tr_gemm<D, 2>(Qs, 32, lane, *(const bf16x8(*)[2]) & db_[2], acc);
                 __builtin_amdgcn_s_setprio(0);
                 tile_barrier();
-                buf = buf == L::NBUF - 1 ? 0 : buf + 1;
                 par ^= 1;
-                if (!had_next) break;
+            };
+            if (MASK) {
+                for (int buf = 0; had_next; buf = buf == L::NBUF - 1 ? 0 : buf + 1) ds_step(buf);
+            } else {
+                for (;;) {
+                    ds_step(std::integral_constant<int, 0>{});
+                    if (!had_next) break;
+                    ds_step(std::integral_constant<int, 1>{});
+                    if (!had_next) break;
+                    ds_step(std::integral_constant<int, 2>{});
+                    if (!had_next) break;
+                }
             }
         }
     };
