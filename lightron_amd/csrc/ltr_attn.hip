@@ -1317,8 +1317,9 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     bool have = c < p.n_chunks;
     if (have) gload(t, 0);
     tile_barrier();
-    int par = 0;
-    while (have) {
+    // one tile; unrolled over the two LDS buffers below, so that LDS addresses are loop-invariant registers plus immediates
+    auto tile_step = [&](auto par_tag) {
+        const int par = par_tag;
         const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
         const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + TILE;
         t++;
@@ -1366,8 +1367,16 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
             __builtin_amdgcn_s_setprio(0);
         }
         tile_barrier();
-        par ^= 1;
         have = have_next;
+    };
+    if (D == 64) {
+        while (have) {
+            tile_step(std::integral_constant<int, 0>{});
+            if (!have) break;
+            tile_step(std::integral_constant<int, 1>{});
+        }
+    } else {   // D = 128 has no registers to spare for the invariant addresses
+        for (int par = 0; have; par ^= 1) tile_step(par);
     }
 
     if (row_ok) {
