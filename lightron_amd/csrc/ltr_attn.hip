@@ -875,6 +875,11 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     const int tile_kpos_lo = pos0 + key0;
     const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
     const bool key_tail = key0 + BN > sk;
+    if (causal) {   // no query of this launch sees the block (a later chunk of the ring): nothing to add, nothing to load
+        int q_lo, q_hi;
+        q_pos_range(0, (int)p.Sq - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], q_lo, q_hi);
+        if (q_hi < tile_kpos_lo) return;
+    }
 
     // resident B operand: K rows for a P wave, V rows for a dS wave; lane (key l32, half hh) holds
     // d = 16*kb + 8*hh .. +7
