@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
 # HBM-side bytes per launch of bwd_dkdv_kernel<128> on config 3, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # command calibrated against streaming kernels of known size (profiles/bench_c3_counters.md)
-DKDV_C3_TRAFFIC_BYTES = 2.10e9
+DKDV_C3_TRAFFIC_BYTES = 2.30e9
 
 
 def _workload(name):
