@@ -325,6 +325,62 @@ __device__ __forceinline__ void lds_tr_gemm(const __bf16 *T, int row0, int lane,
     }
 }
 
+// The same two GEMM loops with the LDS byte addresses of the lane's operands passed in (one per head-dimension block:
+// the swizzle makes them differ per lane, not by a constant) plus an immediate: a kernel that has no registers left to
+// unroll its tile loop over the LDS buffers keeps these addresses in registers and flips them between the buffers with one
+// XOR each per tile, instead of rebuilding every address from pointer + swizzle before each read.
+typedef __attribute__((address_space(3))) const bf16x8 *lds_bf16x8_ptr;
+typedef __attribute__((address_space(3))) i16x4 *lds_i16x4_ptr;
+
+template <int D>
+__device__ __forceinline__ void lds_gemm_pair_at(const unsigned (&addr)[D / 16], int imm_a, int imm_b,
+                                                 const bf16x8 (&ba)[D / 16], const bf16x8 (&bb)[D / 16], f32x16 &ra, f32x16 &rb) {
+    constexpr int NK = D / 16, PF = 2;
+    bf16x8 xa[PF + 1], xb[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        xa[i] = *(lds_bf16x8_ptr)(addr[i] + imm_a);
+        xb[i] = *(lds_bf16x8_ptr)(addr[i] + imm_b);
+    }
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + PF < NK) {
+            xa[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(addr[kb + PF] + imm_a);
+            xb[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(addr[kb + PF] + imm_b);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        ra = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[kb % (PF + 1)], ba[kb], ra, 0, 0, 0);
+        rb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[kb % (PF + 1)], bb[kb], rb, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// addr[j][h]: byte address of the lane's transpose-read element for head-dimension block j, rows +0 (h = 0) / +8 (h = 1)
+template <int D, int NKB>
+__device__ __forceinline__ void lds_tr_gemm_at(const unsigned (&addr)[D / 32][2], int imm, const bf16x8 (&b)[NKB], f32x16 (&acc)[D / 32]) {
+    constexpr int ND = D / 32, N = NKB * ND, PF = 3;
+    auto operand = [&](int i) {
+        const int off = imm + (i / ND) * 16 * D * 2;
+        union {
+            struct { i16x4 a, b; } s;
+            bf16x8 v;
+        } u;
+        u.s.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(addr[i % ND][0] + off));
+        u.s.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(addr[i % ND][1] + off));
+        return u.v;
+    };
+    bf16x8 a[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF && i < N; i++) a[i] = operand(i);
+#pragma unroll
+    for (int step = 0; step < N; step++) {
+        if (step + PF < N) a[(step + PF) % (PF + 1)] = operand(step + PF);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[step / ND], acc[step % ND], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // keys per K / V tile of the forward and dQ kernels
 template <int D>
 struct FwdTile {
@@ -1322,11 +1378,27 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     bool have = c < p.n_chunks;
     if (have) gload(t, 0);
     tile_barrier();
-    // one tile; unrolled over the two LDS buffers below, so that LDS addresses are loop-invariant registers plus immediates
-    auto tile_step = [&](auto par_tag) {
-        const int par = par_tag;
+    // LDS byte addresses of this lane's operands in the K tile of the current buffer (the V tile and the other 32-key
+    // blocks are immediates away): kept in registers and flipped to the other buffer with one XOR each per tile
+    static_assert((BUF_ELEMS * 2 & (BUF_ELEMS * 2 - 1)) == 0, "buffer size must be a power of two for the XOR flip");
+    unsigned pa[D / 16], ta[D / 32][2];
+    {
+        const unsigned lds0 = lds_address(smem);   // the only LDS object of the kernel: aligned far beyond the buffer size
+        const int sw = lds_swz<D>(l32) ^ hh;        // rows l32 + 32 n share the swizzle word of row l32
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) pa[kb] = lds0 + ((l32 * D + (((2 * kb) ^ sw) << 3)) << 1);
+        const int li = lane & 15, g = lane >> 4;
+#pragma unroll
+        for (int j = 0; j < D / 32; j++)
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int col = j * 32 + ((g & 1) << 4) + ((li & 3) << 2), row = 4 * (g >> 1) + (li >> 2) + 8 * e;
+                ta[j][e] = lds0 + ((lds_swz_off<D>(row, col >> 3) + (col & 7)) << 1);
+            }
+    }
+    int par = 0;
+    while (have) {
         const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
-        const __bf16 *Ks = (const __bf16 *)smem + par * BUF_ELEMS, *Vs = Ks + TILE;
         t++;
         settle();
         const bool have_next = c < p.n_chunks;
@@ -1338,9 +1410,8 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
         for (int nb = 0; nb < BN / 32; nb++) {
             f32x16 s = zero16, dp = zero16;
-            const int sw = lds_swz<D>(nb * 32 + l32) ^ hh;       // chunk 2*kb + hh lives at (2*kb) ^ sw
             __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
-            lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, sw, Vs + (nb * 32 + l32) * D, sw, qreg, doreg, s, dp);
+            lds_gemm_pair_at<D>(pa, nb * 32 * D * 2, TILE * 2 + nb * 32 * D * 2, qreg, doreg, s, dp);
             __builtin_amdgcn_s_setprio(0);
             // mask fix-up (tail of the chunk, diagonal tiles, rows past the end): wave-uniform branch touching S only;
             // an invisible entry gets S = -inf, so P = 0 and dS = 0
@@ -1367,21 +1438,20 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
             __builtin_amdgcn_s_setprio(1);
             {
                 const bf16x8 dsb[2] = {operand_of(ds, 0), operand_of(ds, 1)};
-                lds_tr_gemm<D, 2>(Ks, nb * 32, lane, dsb, dqacc);   // 16 keys per MFMA
+                lds_tr_gemm_at<D, 2>(ta, nb * 32 * D * 2, dsb, dqacc);   // 16 keys per MFMA
             }
             __builtin_amdgcn_s_setprio(0);
         }
         tile_barrier();
-        have = have_next;
-    };
-    if (D == 64) {
-        while (have) {
-            tile_step(std::integral_constant<int, 0>{});
-            if (!have) break;
-            tile_step(std::integral_constant<int, 1>{});
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) pa[kb] ^= BUF_ELEMS * 2;
+#pragma unroll
+        for (int j = 0; j < D / 32; j++) {
+            ta[j][0] ^= BUF_ELEMS * 2;
+            ta[j][1] ^= BUF_ELEMS * 2;
         }
-    } else {   // D = 128 has no registers to spare for the invariant addresses
-        for (int par = 0; have; par ^= 1) tile_step(par);
+        par ^= 1;
+        have = have_next;
     }
 
     if (row_ok) {
