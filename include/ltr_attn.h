@@ -160,7 +160,8 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_split;
     float scale;
     uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O */
-    int32_t io_dtype;     /* LTR_BF16 (the backward kernels are bf16 only) */
+    int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: scalar fp32 kernels for the 1e-4 parity cases;
+                             LTR_DQ_BF16 and LTR_DELTA_FROM_O are bf16 only and return LTR_EUNSUP with it) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
     const void *o;        /* forward output, bf16, only read with LTR_DELTA_FROM_O */

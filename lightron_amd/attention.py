@@ -225,15 +225,16 @@ class BlockAttentionFunction(torch.autograd.Function):
         q, o, lse, *kv = ctx.saved_tensors
         n_chunks, k_pos0, q_pos0, q_split, causal, scale = ctx.meta
         ks, vs = kv[:n_chunks], kv[n_chunks:]
-        if q.dtype != torch.bfloat16:
-            raise RuntimeError("the HIP backward is implemented for bf16 inputs")
+        if q.dtype not in (torch.bfloat16, torch.float32):
+            raise RuntimeError("the HIP backward is implemented for bf16 and fp32 inputs")
+        f32 = q.dtype == torch.float32
         if do.stride(3) != 1:
             do = do.contiguous()
         do = do.to(q.dtype)
-        fuse = o.dtype == torch.bfloat16            # DELTA computed by the dQ kernel from o
+        fuse = o.dtype == torch.bfloat16 and not f32   # DELTA computed by the dQ kernel from o
         delta = (torch.empty(lse.shape, dtype=torch.float32, device=q.device) if fuse else attn_delta(o, do))
         # one launch sees every chunk: dQ is written as bf16 by the kernel; otherwise it accumulates in fp32
-        direct = n_chunks <= _lib.LTR_MAX_CHUNKS
+        direct = n_chunks <= _lib.LTR_MAX_CHUNKS and not f32
         dq_acc = (torch.empty(q.shape, dtype=torch.bfloat16, device=q.device) if direct
                   else torch.zeros(q.shape, dtype=torch.float32, device=q.device))
         # one fp32 buffer per gradient, sliced along the sequence: every chunk's accumulator has the same strides
@@ -246,8 +247,11 @@ class BlockAttentionFunction(torch.autograd.Function):
         dv_accs = [dv_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale,
                             o=o if fuse else None)
-        dq = dq_acc if direct else cast_to_bf16(dq_acc)
-        dk16, dv16 = cast_to_bf16(dk_buf), cast_to_bf16(dv_buf)
+        if f32:   # the fp32 kernels accumulate into the gradients themselves
+            dq, dk16, dv16 = dq_acc, dk_buf, dv_buf
+        else:
+            dq = dq_acc if direct else cast_to_bf16(dq_acc)
+            dk16, dv16 = cast_to_bf16(dk_buf), cast_to_bf16(dv_buf)
         dks = [dk16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         dvs = [dv16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         return (dq, None, None, None, None, None, None, None, None, *dks, *dvs)

@@ -1483,6 +1483,206 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     }
 }
 
+// ------------------------------------------------------------------------------ backward, fp32
+// The fp32 path (1e-4 parity cases, not a performance path): scalar FMAs like fwd_f32_kernel, no atomics.
+//   bwd_dq_f32_kernel    one query row per lane (q, dO, dQ in registers), K/V tiles of 32 keys broadcast from LDS
+//   bwd_dkdv_f32_kernel  one key per lane, Q/dO tiles of 32 rows (+ LSE, DELTA) broadcast from LDS; two passes so that
+//                        the per-lane state fits the register file: DV = false keeps K, V, dK; DV = true keeps K, dV
+template <int D>
+__global__ __launch_bounds__(64) void bwd_dq_f32_kernel(const BwdParams p) {
+    constexpr int BN = 32;
+    __shared__ __attribute__((aligned(16))) float Ks[BN * D];
+    __shared__ __attribute__((aligned(16))) float Vs[BN * D];
+    const int tid = threadIdx.x;
+    const bool causal = p.flags & LTR_CAUSAL;
+    const int n_qt = (p.Sq + 63) / 64;
+    const int qt = n_qt - 1 - (int)(blockIdx.x % n_qt), bh = blockIdx.x / n_qt;
+    const int b = bh / p.Hq, h = bh % p.Hq, hkv = h / p.n_rep;
+    const int row0 = qt * 64, my_row = row0 + tid;
+    const bool row_ok = my_row < p.Sq;
+    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int blk_lo, blk_hi;
+    q_pos_range(row0, min(row0 + 64, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+
+    // the accumulator covers 64 (D = 128: 32) elements of the head dimension at a time, one pass over the keys each, so that the
+    // per-lane state stays inside the register file
+    constexpr int DP = D == 128 ? 32 : 64;
+    float q[D], dO[D], dq[DP];
+    float lse = INFINITY, dlt = 0.f;   // +inf: P = exp(s - inf) = 0 for rows past the end and rows that saw no key
+    {
+        const int rs = min(my_row, p.Sq - 1);
+        const float *qp = (const float *)p.q + b * p.qs[0] + (long long)rs * p.qs[1] + h * p.qs[2];
+        const float *dop = (const float *)p.d_o + b * p.dos[0] + (long long)rs * p.dos[1] + h * p.dos[2];
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            q[d] = qp[d];
+            dO[d] = dop[d];
+        }
+        if (row_ok) {
+            const float l = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row];
+            lse = l == -INFINITY ? INFINITY : l;
+            dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
+        }
+    }
+    for (int part = 0; part < D / DP; part++) {
+#pragma unroll
+    for (int d = 0; d < DP; d++) dq[d] = 0.f;
+    for (int c = 0; c < p.n_chunks; c++) {
+        const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
+        const int nvis = causal ? max(0, min(sk, blk_hi - pos0 + 1)) : sk;
+        const float *kp = (const float *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+        const float *vp = (const float *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+        for (int key0 = 0; key0 < nvis; key0 += BN) {
+            __syncthreads();
+            for (int i = tid; i < BN * D / 4; i += 64) {
+                const int key = key0 + i / (D / 4), dc = i % (D / 4);
+                f32x4 kv = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
+                if (key < sk) {
+                    kv = *(const f32x4 *)(kp + (long long)key * p.ks[1] + dc * 4);
+                    vv = *(const f32x4 *)(vp + (long long)key * p.vs[1] + dc * 4);
+                }
+                *(f32x4 *)(Ks + i * 4) = kv;
+                *(f32x4 *)(Vs + i * 4) = vv;
+            }
+            __syncthreads();
+#pragma unroll 1
+            for (int j = 0; j < BN; j++) {
+                float s = 0.f, dp = 0.f;
+#pragma unroll
+                for (int d4 = 0; d4 < D / 4; d4++) {
+                    const f32x4 kq = *(const f32x4 *)(Ks + j * D + 4 * d4), vq = *(const f32x4 *)(Vs + j * D + 4 * d4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        s = fmaf(q[4 * d4 + e], kq[e], s);
+                        dp = fmaf(dO[4 * d4 + e], vq[e], dp);
+                    }
+                    if ((d4 & 7) == 7) asm volatile("" ::: "memory");   // bounds the LDS reads in flight (registers)
+                }
+                const int key = key0 + j;
+                const bool vis = key < sk && (!causal || pos0 + key <= my_pos);
+                const float pj = vis ? expf(s * p.scale - lse) : 0.f;
+                const float ds = pj * (dp - dlt);
+#pragma unroll
+                for (int d = 0; d < DP; d++) dq[d] = fmaf(ds, Ks[j * D + part * DP + d], dq[d]);
+            }
+        }
+    }
+    if (row_ok) {
+        float *dqp = (float *)p.dq + b * p.dqs[0] + (long long)my_row * p.dqs[1] + h * p.dqs[2] + part * DP;
+#pragma unroll
+        for (int d = 0; d < DP; d++) dqp[d] += dq[d] * p.scale;
+    }
+    }
+}
+
+template <int D, bool DV>
+__global__ __launch_bounds__(64) void bwd_dkdv_f32_kernel(const BwdParams p) {
+    constexpr int BM = 32;
+    __shared__ __attribute__((aligned(16))) float Qs[BM * D];
+    __shared__ __attribute__((aligned(16))) float dOs[BM * D];
+    __shared__ float lse_s[BM], dlt_s[BM];
+    const int tid = threadIdx.x;
+    const bool causal = p.flags & LTR_CAUSAL;
+    // block -> (batch, kv head, chunk, 64-key tile)
+    const int P = p.B * p.Hkv;
+    const int pair = blockIdx.x % P;
+    int kt = blockIdx.x / P;
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv;
+    int c = 0;
+    for (; c < p.n_chunks; c++) {
+        const int n = (p.chunk[c].sk + 63) / 64;
+        if (kt < n) break;
+        kt -= n;
+    }
+    if (c >= p.n_chunks) return;
+    const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
+    const int my_key = kt * 64 + tid;
+    const bool key_ok = my_key < sk;
+    const int my_kpos = pos0 + my_key, tile_kpos_lo = pos0 + kt * 64;
+
+    constexpr int DP = D == 128 ? 32 : 64;   // see bwd_dq_f32_kernel
+    float k[D], v[DV ? 1 : D], acc[DP];
+    {
+        const int ks_ = min(my_key, sk - 1);
+        const float *kp = (const float *)p.chunk[c].k + b * p.ks[0] + (long long)ks_ * p.ks[1] + hkv * p.ks[2];
+        const float *vp = (const float *)p.chunk[c].v + b * p.vs[0] + (long long)ks_ * p.vs[1] + hkv * p.vs[2];
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            k[d] = kp[d];
+            if (!DV) v[d] = vp[d];
+        }
+    }
+    for (int part = 0; part < D / DP; part++) {
+#pragma unroll
+    for (int d = 0; d < DP; d++) acc[d] = 0.f;
+    for (int rep = 0; rep < p.n_rep; rep++) {
+        const int h = hkv * p.n_rep + rep;
+        const float *qp = (const float *)p.q + b * p.qs[0] + h * p.qs[2];
+        const float *dop = (const float *)p.d_o + b * p.dos[0] + h * p.dos[2];
+        const long long so = ((long long)b * p.Hq + h) * p.Sq;
+        for (int row0 = 0; row0 < p.Sq; row0 += BM) {
+            if (causal) {   // no row of the tile sees any key of the block
+                int lo, hi;
+                q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
+                if (hi < tile_kpos_lo) continue;
+            }
+            __syncthreads();
+            for (int i = tid; i < BM * D / 4; i += 64) {
+                const int row = row0 + i / (D / 4), dc = i % (D / 4);
+                f32x4 qv = {0.f, 0.f, 0.f, 0.f}, dv = {0.f, 0.f, 0.f, 0.f};
+                if (row < p.Sq) {
+                    qv = *(const f32x4 *)(qp + (long long)row * p.qs[1] + dc * 4);
+                    dv = *(const f32x4 *)(dop + (long long)row * p.dos[1] + dc * 4);
+                }
+                *(f32x4 *)(Qs + i * 4) = qv;
+                *(f32x4 *)(dOs + i * 4) = dv;
+            }
+            if (tid < BM) {
+                const int row = row0 + tid;
+                const float l = row < p.Sq ? p.lse[so + row] : INFINITY;
+                lse_s[tid] = l == -INFINITY ? INFINITY : l;     // +inf: P = 0
+                dlt_s[tid] = row < p.Sq ? p.delta[so + row] : 0.f;
+            }
+            __syncthreads();
+#pragma unroll 1
+            for (int i = 0; i < BM; i++) {
+                float s = 0.f, dp = 0.f;
+#pragma unroll
+                for (int d4 = 0; d4 < D / 4; d4++) {
+                    const f32x4 qq = *(const f32x4 *)(Qs + i * D + 4 * d4);
+                    f32x4 oq = {0.f, 0.f, 0.f, 0.f};
+                    if (!DV) oq = *(const f32x4 *)(dOs + i * D + 4 * d4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        s = fmaf(k[4 * d4 + e], qq[e], s);
+                        if (!DV) dp = fmaf(v[4 * d4 + e], oq[e], dp);
+                    }
+                    if ((d4 & 7) == 7) asm volatile("" ::: "memory");   // bounds the LDS reads in flight (registers)
+                }
+                const int qpos = q_position(row0 + i, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+                const bool vis = key_ok && (!causal || my_kpos <= qpos);
+                const float pi = vis ? expf(s * p.scale - lse_s[i]) : 0.f;
+                if (DV) {
+#pragma unroll
+                    for (int d = 0; d < DP; d++) acc[d] = fmaf(pi, dOs[i * D + part * DP + d], acc[d]);
+                } else {
+                    const float ds = pi * (dp - dlt_s[i]);
+#pragma unroll
+                    for (int d = 0; d < DP; d++) acc[d] = fmaf(ds, Qs[i * D + part * DP + d], acc[d]);
+                }
+            }
+        }
+    }
+    if (key_ok) {
+        float *gp = (DV ? p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2]
+                        : p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2]) + part * DP;
+        const float mul = DV ? 1.f : p.scale;
+#pragma unroll
+        for (int d = 0; d < DP; d++) gp[d] += acc[d] * mul;
+    }
+    }
+}
+
 // ------------------------------------------------------------------------------ host side
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -1664,12 +1864,15 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     const bool fused_delta = a->flags & LTR_DELTA_FROM_O;
     if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
-    if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;
+    if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
+    const bool f32 = a->io_dtype == LTR_F32;
+    if (f32 && (a->flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O))) return LTR_EUNSUP;   // bf16 conveniences only
+    const int eb = f32 ? 4 : 2;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
     if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
     if (!aligned16(a->q) || !aligned16(a->d_o) || (do_dq && !aligned16(a->dq))) return LTR_EALIGN;
-    if (!strides_ok(a->q_stride, 2) || !strides_ok(a->do_stride, 2) || !strides_ok(a->k_stride, 2) ||
-        !strides_ok(a->v_stride, 2) || !strides_ok(a->dk_stride, 4) || !strides_ok(a->dv_stride, 4))
+    if (!strides_ok(a->q_stride, eb) || !strides_ok(a->do_stride, eb) || !strides_ok(a->k_stride, eb) ||
+        !strides_ok(a->v_stride, eb) || !strides_ok(a->dk_stride, 4) || !strides_ok(a->dv_stride, 4))
         return LTR_EALIGN;
     for (int i = 0; i < 3; i++)
         if (a->dq_stride[i] < 0) return LTR_EINVAL;
@@ -1729,6 +1932,26 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     const long long nblk = tiles * p.B * p.Hkv;
     if (nblk > 0x7fffffffLL) return LTR_EINVAL;
     hipStream_t st = (hipStream_t)stream;
+    if (f32) {
+        long long tiles64 = 0;
+        for (int c = 0; c < a->n_chunks; c++) tiles64 += (a->chunk[c].sk + 63) / 64;
+        const long long nq = (long long)((p.Sq + 63) / 64) * p.B * p.Hq, nk = tiles64 * p.B * p.Hkv;
+        if (nq > 0x7fffffffLL || nk > 0x7fffffffLL) return LTR_EINVAL;
+        if (a->D == 128) {
+            if (do_dq) hipLaunchKernelGGL(bwd_dq_f32_kernel<128>, dim3((unsigned)nq), dim3(64), 0, st, p);
+            if (do_dkdv) {
+                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<128, false>), dim3((unsigned)nk), dim3(64), 0, st, p);
+                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<128, true>), dim3((unsigned)nk), dim3(64), 0, st, p);
+            }
+        } else {
+            if (do_dq) hipLaunchKernelGGL(bwd_dq_f32_kernel<64>, dim3((unsigned)nq), dim3(64), 0, st, p);
+            if (do_dkdv) {
+                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<64, false>), dim3((unsigned)nk), dim3(64), 0, st, p);
+                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<64, true>), dim3((unsigned)nk), dim3(64), 0, st, p);
+            }
+        }
+        return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    }
     rc = enable_large_lds();
     if (rc) return rc;
     const long long nblk_q = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;

@@ -113,13 +113,15 @@ def test_config2_shape_scaled_multi_chunk_bf16(ltr):
         assert (ring.last_lse.cpu().double() - rlse).abs().max() < LSE_TOL_BF16
 
 
-def _grads_case(ltr, B, Hq, Hkv, D, S, W, layout, causal, seed, dist="normal"):
+def _grads_case(ltr, B, Hq, Hkv, D, S, W, layout, causal, seed, dist="normal", dtype=torch.bfloat16):
     """Every rank of a ring: forward and backward, dK/dV summed over ranks, vs dense autograd."""
     g = torch.Generator().manual_seed(seed)
     if dist == "normal":
-        mk = lambda shape: _randn(shape, g, torch.bfloat16)
+        mk = lambda shape: _randn(shape, g, dtype)
     else:
-        mk = lambda shape: (torch.rand(shape, generator=g) * 2 - 1).to(torch.bfloat16)
+        mk = lambda shape: (torch.rand(shape, generator=g) * 2 - 1).to(dtype)
+    o_tol, lse_tol, g_tol = ((O_TOL_BF16, LSE_TOL_BF16, GRAD_RTOL_BF16) if dtype == torch.bfloat16
+                             else (F32_TOL, F32_TOL, F32_TOL))
     q, k, v, do = mk((B, S, Hq, D)), mk((B, S, Hkv, D)), mk((B, S, Hkv, D)), mk((B, S, Hq, D))
     pos = torch.arange(S)
     ro, rlse, rdq, rdk, rdv = orc.dense_attention_grads(q, k, v, do, pos, pos, causal)
@@ -146,10 +148,13 @@ def _grads_case(ltr, B, Hq, Hkv, D, S, W, layout, causal, seed, dist="normal"):
     for r in range(W):
         dk[:, rank_pos[r].cuda()] = kl[r].grad
         dv[:, rank_pos[r].cuda()] = vl[r].grad
-    assert (o.cpu().double() - ro).abs().max() < O_TOL_BF16
-    assert (lse.double() - rlse).abs().max() < LSE_TOL_BF16
+    assert (o.cpu().double() - ro).abs().max() < o_tol
+    assert (lse.double() - rlse).abs().max() < lse_tol
     for name, a, b in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
-        assert _rel(a.cpu(), b) < GRAD_RTOL_BF16, (name, _rel(a.cpu(), b))
+        assert a.dtype == dtype
+        assert _rel(a.cpu(), b) < g_tol, (name, _rel(a.cpu(), b))
+        if dtype == torch.float32:
+            assert (a.cpu().double() - b).abs().max() < F32_TOL * max(1.0, b.abs().max().item()), name
 
 
 def test_config3_shape_scaled_gqa_zigzag_fwd_bwd(ltr):
@@ -164,6 +169,62 @@ def test_contiguous_ring_mha_fwd_bwd(ltr):
 def test_noncausal_d64_fwd_bwd(ltr):
     """Config 5's kernel case at reduced size: non-causal, D=64, U(-1,1), seed 7."""
     _grads_case(ltr, 2, 4, 4, 64, 384, 1, "contiguous", False, 7, dist="uniform")
+
+
+def test_config1_fp32_ring_fwd_bwd(ltr):
+    """Config 1's shape (B=2, H=8, S=1024 as 4 ranks x 256, D=64, fp32, causal) through the fp32 backward kernels:
+    O, LSE and all three gradients to 1e-4."""
+    _grads_case(ltr, 2, 8, 8, 64, 1024, 4, "contiguous", True, 0, dtype=torch.float32)
+
+
+def test_fp32_gqa_zigzag_d128_fwd_bwd(ltr):
+    _grads_case(ltr, 1, 4, 2, 128, 512, 4, "zigzag", True, 5, dtype=torch.float32)
+
+
+def test_fp32_noncausal_fwd_bwd(ltr):
+    _grads_case(ltr, 2, 2, 1, 64, 192, 1, "contiguous", False, 9, dist="uniform", dtype=torch.float32)
+
+
+@pytest.mark.parametrize("seed", list(range(10)))
+def test_fp32_backward_random_shapes(ltr, seed):
+    """Ragged sizes, several KV chunks with gaps in their positions, GQA, rows that see no key: the fp32 backward against
+    dense fp64 autograd, 1e-4 relative per tensor."""
+    import random
+    rnd = random.Random(9000 + seed)
+    g = torch.Generator().manual_seed(9500 + seed)
+    D = rnd.choice([64, 128])
+    Hkv = rnd.choice([1, 2])
+    Hq = Hkv * rnd.choice([1, 3])
+    B = rnd.choice([1, 2])
+    Sq = rnd.choice([1, 31, 64, 65, 100, 150])
+    n_ch = rnd.randint(1, 3)
+    sks = [rnd.choice([1, 17, 64, 70, 129]) for _ in range(n_ch)]
+    causal = rnd.random() < 0.7
+    starts, p = [], rnd.randint(0, 20)
+    for sk in sks:
+        starts.append(p)
+        p += sk + rnd.choice([0, 0, 5])
+    qp = rnd.randint(0, p)
+    q_pos = torch.arange(qp, qp + Sq)
+    q, do = _randn((B, Sq, Hq, D), g, torch.float32), _randn((B, Sq, Hq, D), g, torch.float32)
+    kbuf, vbuf = _randn((B, sum(sks), Hkv, D), g, torch.float32), _randn((B, sum(sks), Hkv, D), g, torch.float32)
+    offs = [sum(sks[:i]) for i in range(n_ch)]
+    k_pos = torch.cat([torch.arange(starts[i], starts[i] + sks[i]) for i in range(n_ch)])
+    ro, rlse, rdq, rdk, rdv = orc.dense_attention_grads(q, kbuf, vbuf, do, q_pos, k_pos, causal)
+    qd = q.cuda().requires_grad_(True)
+    kd, vd = kbuf.cuda().requires_grad_(True), vbuf.cuda().requires_grad_(True)
+    ks = [kd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    vs = [vd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    o, lse = ltr.block_attention(qd, ks, vs, starts, qp, None, causal=causal)
+    o.backward(do.cuda())
+    assert (o.detach().cpu().double() - ro).abs().max() < F32_TOL
+    for name, a, b in (("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        assert a.dtype == torch.float32
+        assert torch.isfinite(a).all(), name
+        if b.abs().max() > 0:
+            assert _rel(a.cpu(), b) < F32_TOL, (name, _rel(a.cpu(), b))
+        else:
+            assert a.abs().max() == 0, name
 
 
 def test_ragged_bwd(ltr):
