@@ -25,6 +25,10 @@
 //                        (same direct-to-LDS tiles as the forward), recomputes S and dP and
 //                        accumulates dQ^T in registers.  No atomics anywhere: results are
 //                        bitwise reproducible.
+//   bwd_dq_f32_kernel<D>, bwd_dkdv_f32_kernel<D, DV>
+//                        the same backward in scalar fp32 (no MFMA), for the 1e-4 parity cases.
+//   The tile loops of the bf16 kernels are unrolled over their LDS buffers (or, where registers are short,
+//   keep per-lane LDS addresses in registers): no address arithmetic is left between the MFMAs.
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, i = l % 32, h = l / 32):
 //   A[i][8h .. 8h+7], B[8h .. 8h+7][i], C[8*(r/4) + 4h + r%4][i] for accumulator register r.
@@ -136,27 +140,6 @@ __device__ __forceinline__ i16x4 lds_read_tr16(const __bf16 *p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 __attribute__((address_space(3))) *)(p));
 }
 
-// 8 K-dim values for an MFMA operand whose K index runs over the ROWS of a row-major LDS
-// tile: rows {k0 + 4h + 0..3} and {k0 + 8 + 4h + 0..3} at column n_base + (l % 32).
-// This row set is the one the accumulator registers 8b..8b+7 of a 32x32 MFMA result
-// hold (rows 16b + 4h + 0..3 and 16b + 8 + 4h + 0..3), so a result tile can feed the
-// next GEMM as an operand without leaving registers.
-__device__ __forceinline__ bf16x8 lds_operand_tr(const __bf16 *tile, int stride, int k0, int n_base, int lane) {
-    const int li = lane & 15, g = lane >> 4;
-    const int hh = g >> 1;
-    const int col = n_base + ((g & 1) << 4) + ((li & 3) << 2);
-    const int row = k0 + 4 * hh + (li >> 2);
-    i16x4 lo = lds_read_tr16(tile + row * stride + col);
-    i16x4 hi = lds_read_tr16(tile + (row + 8) * stride + col);
-    union {
-        struct { i16x4 a, b; } s;
-        bf16x8 v;
-    } u;
-    u.s.a = lo;
-    u.s.b = hi;
-    return u.v;
-}
-
 // Unpadded row-major LDS tile of D bf16 per row whose 16-byte chunks are XOR-swizzled: chunk c of row r
 // lives at chunk position c ^ lds_swz<D>(r).  LDS has 64 banks of 4 bytes; a 128-bit read is served 16
 // lanes at a time and a 64-bit (transpose) read 32 lanes at a time.  With this permutation both the MFMA
@@ -172,7 +155,12 @@ __device__ __forceinline__ int lds_swz_off(int row, int chunk) {   // element of
     return row * D + ((chunk ^ lds_swz<D>(row)) << 3);
 }
 
-// transpose-read operand (same contract as lds_operand_tr) from a swizzled tile
+// 8 K-dim values for an MFMA operand whose K index runs over the ROWS of a row-major LDS
+// tile: rows {k0 + 4h + 0..3} and {k0 + 8 + 4h + 0..3} at column n_base + (l % 32).
+// This row set is the one the accumulator registers 8b..8b+7 of a 32x32 MFMA result
+// hold (rows 16b + 4h + 0..3 and 16b + 8 + 4h + 0..3), so a result tile can feed the
+// next GEMM as an operand without leaving registers.
+// (tile = swizzled tile, see lds_swz)
 template <int D>
 __device__ __forceinline__ bf16x8 lds_operand_tr_swz(const __bf16 *tile, int k0, int n_base, int lane) {
     const int li = lane & 15, g = lane >> 4;
@@ -218,13 +206,6 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) {
     union { uint4 u; bf16x8 v; } c;
     c.u = x;
     return c.v;
-}
-
-__device__ __forceinline__ bf16x8 pack_bf16x8(const f32x16 &s, int base) {
-    bf16x8 r;
-#pragma unroll
-    for (int e = 0; e < 8; e++) r[e] = (__bf16)s[base + e];
-    return r;
 }
 
 struct PackedTile {   // 16 bf16 values of one lane's 32x32 tile column, as the two B operands of K = 16
@@ -339,14 +320,14 @@ __device__ __forceinline__ void lds_gemm_pair_at(const unsigned (&addr)[D / 16],
     bf16x8 xa[PF + 1], xb[PF + 1];
 #pragma unroll
     for (int i = 0; i < PF; i++) {
-        xa[i] = *(lds_bf16x8_ptr)(addr[i] + imm_a);
-        xb[i] = *(lds_bf16x8_ptr)(addr[i] + imm_b);
+        xa[i] = *(lds_bf16x8_ptr)(uintptr_t)(addr[i] + imm_a);
+        xb[i] = *(lds_bf16x8_ptr)(uintptr_t)(addr[i] + imm_b);
     }
 #pragma unroll
     for (int kb = 0; kb < NK; kb++) {
         if (kb + PF < NK) {
-            xa[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(addr[kb + PF] + imm_a);
-            xb[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(addr[kb + PF] + imm_b);
+            xa[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(uintptr_t)(addr[kb + PF] + imm_a);
+            xb[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(uintptr_t)(addr[kb + PF] + imm_b);
         }
         __builtin_amdgcn_sched_barrier(0);
         ra = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[kb % (PF + 1)], ba[kb], ra, 0, 0, 0);
@@ -365,8 +346,8 @@ __device__ __forceinline__ void lds_tr_gemm_at(const unsigned (&addr)[D / 32][2]
             struct { i16x4 a, b; } s;
             bf16x8 v;
         } u;
-        u.s.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(addr[i % ND][0] + off));
-        u.s.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(addr[i % ND][1] + off));
+        u.s.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(addr[i % ND][0] + off));
+        u.s.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(addr[i % ND][1] + off));
         return u.v;
     };
     bf16x8 a[PF + 1];
@@ -892,7 +873,7 @@ __device__ __forceinline__ unsigned bwd_ds_pair(unsigned pu, const f32x16 &dpm, 
 template <int D>
 __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     using L = BwdLds<D>;
-    constexpr int BN = L::BN, BM = L::BM, NT = L::NT;
+    constexpr int BN = L::BN, BM = L::BM;
     constexpr int CPR = D / 8;
     constexpr int RPI = 64 / CPR;        // rows filled by one wave-wide LDS-direct load (1 KB)
     constexpr int NI = BM / (RPI * 8);   // such loads per wave, per tensor and per tile
@@ -1147,7 +1128,11 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             };
             static_assert(L::NBUF == 3, "unrolled over three buffers");
             if (MASK) {
-                for (int buf = 0; more; buf = buf == L::NBUF - 1 ? 0 : buf + 1) p_step(buf);
+                int buf = 0;
+                while (more) {
+                    p_step(buf);
+                    buf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                }
             } else {
                 for (;;) {
                     p_step(std::integral_constant<int, 0>{});
@@ -1216,7 +1201,11 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 par ^= 1;
             };
             if (MASK) {
-                for (int buf = 0; had_next; buf = buf == L::NBUF - 1 ? 0 : buf + 1) ds_step(buf);
+                int buf = 0;
+                while (had_next) {
+                    ds_step(buf);
+                    buf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                }
             } else {
                 for (;;) {
                     ds_step(std::integral_constant<int, 0>{});
