@@ -516,6 +516,9 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             for (int j = 0; j < 2 * NI; j++) gload_one(j, t, par ^ 1);
         }
 
+        // A wave whose 32 rows all precede the tile's first key (upper part of a diagonal tile, rows past the end) has
+        // nothing to add: it only takes part in the transfers and the barrier.
+        if (!causal || pos0 + key0 <= w_hi) {
         // S^T of the two 32-key blocks of the tile.  The wave raises its priority while it issues MFMAs: the
         // other wave of the SIMD then fills the gaps with its softmax arithmetic instead of delaying them.
         __builtin_amdgcn_s_setprio(1);
@@ -605,6 +608,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             lds_tr_gemm<D, 2 * NB>(Vs, 0, lane, pb, oacc);   // 16 keys per MFMA
         }
         __builtin_amdgcn_s_setprio(0);
+        }
         tile_barrier();
         have = have_next;
     };
@@ -1395,7 +1399,9 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
 
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         // 32 keys at a time, one block after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
-        // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic
+        // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic.  A wave whose rows all
+        // precede the tile's first key has nothing to add (see the forward kernel).
+        if (!causal || pos0 + key0 <= w_hi) {
 #pragma unroll
         for (int nb = 0; nb < BN / 32; nb++) {
             f32x16 s = zero16, dp = zero16;
@@ -1430,6 +1436,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
                 lds_tr_gemm_at<D, 2>(ta, nb * 32 * D * 2, dsb, dqacc);   // 16 keys per MFMA
             }
             __builtin_amdgcn_s_setprio(0);
+        }
         }
         tile_barrier();
 #pragma unroll
