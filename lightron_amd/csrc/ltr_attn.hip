@@ -46,6 +46,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 #define LTR_LOG2E 1.4426950408889634f
 #define LTR_LN2 0.6931471805599453f
@@ -828,14 +829,15 @@ __global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst
 //   bwd_dq_kernel    a block owns 256 query rows of one query head (32 per wave; Q and dO
 //                    operands in registers), loops over 64-key K/V tiles like the forward;
 //                    dQ^T accumulates in registers.
-// LDS of bwd_dkdv_kernel (dynamic): three buffers of {Q tile, dO tile, LSE*log2e, -DELTA}, the P slots, the tile lists.
+// LDS of bwd_dkdv_kernel (dynamic): three buffers of {Q tile, dO tile, -LSE/scale, -DELTA, row positions}, the P slots,
+// the tile lists.
 template <int D>
 struct BwdLds {
     static constexpr int BN = 128;      // keys per block, 32 per wave pair
     static constexpr int BM = 64;       // query rows per tile (two 32-row MFMA sub-tiles)
     static constexpr int NT = 512;      // threads per block
     static constexpr int TILE = BM * D;                                  // elements; rows unpadded, chunks swizzled
-    static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BM * 4;          // Q, dO, LSE*log2e, -DELTA
+    static constexpr int BUF_BYTES = 2 * TILE * 2 + 3 * BM * 4;          // Q, dO, -LSE/scale, -DELTA, row positions (masked tiles)
     static constexpr int P_SLOT = 64 * 32;                               // one lane = 16 bf16 = 32 bytes
     static constexpr int NBUF = 3;                                       // tile t (P waves), t-1 (dS waves), t+1 (in flight)
     static constexpr int P_OFF = NBUF * BUF_BYTES;
@@ -844,25 +846,20 @@ struct BwdLds {
     static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;     // two tile lists (ushort) + counts
 };
 
-struct BwdMaskCtx {
-    bool key_ok, causal;
-    int my_kpos, row_base, Sq, q_split, p0, p1;
-};
-
-__device__ __forceinline__ bool bwd_visible(const BwdMaskCtx &m, int r0, int r, int hh) {
-    const int qrow = m.row_base + r0 + 8 * (r / 4) + 4 * hh + (r % 4);
-    const int qpos = q_position(qrow, m.q_split, m.p0, m.p1);
-    return m.key_ok && qrow < m.Sq && (!m.causal || m.my_kpos <= qpos);
-}
+// Masked tiles: the visibility of (row, key) is kpos <= qpos[row], with the rows' positions staged in LDS beside LSE and
+// DELTA (INT_MIN for a row past the end; INT_MAX - 1 for every row when there is no causal mask) and kpos = INT_MAX for
+// a key past the end of its chunk: one compare and one select per element, whatever the position map of the rows is.
+constexpr int BWD_QPOS_NONE = (int)0x80000000, BWD_QPOS_ALL = 0x7ffffffe, BWD_KPOS_NONE = 0x7fffffff;
 
 // P wave, accumulator registers 2j and 2j+1 of a 32x32 sub-tile: sm = S - LSE / scale (the accumulator started at
-// -LSE / scale), P = exp2(sm * c2) -> one packed bf16 pair in accumulator layout
+// -LSE / scale), P = exp2(sm * c2) -> one packed bf16 pair in accumulator layout; qpos = positions of the sub-tile's 16
+// rows in accumulator-register order
 template <bool MASK>
-__device__ __forceinline__ unsigned bwd_p_pair(const f32x16 &sm, int j, int r0, int hh, float c2, const BwdMaskCtx &m) {
+__device__ __forceinline__ unsigned bwd_p_pair(const f32x16 &sm, int j, float c2, int kpos, const int (&qpos)[16]) {
     float p0 = __builtin_amdgcn_exp2f(sm[2 * j] * c2), p1 = __builtin_amdgcn_exp2f(sm[2 * j + 1] * c2);
     if (MASK) {
-        p0 = bwd_visible(m, r0, 2 * j, hh) ? p0 : 0.f;
-        p1 = bwd_visible(m, r0, 2 * j + 1, hh) ? p1 : 0.f;
+        p0 = kpos <= qpos[2 * j] ? p0 : 0.f;
+        p1 = kpos <= qpos[2 * j + 1] ? p1 : 0.f;
     }
     return pack2_bf16(p0, p1);
 }
@@ -985,6 +982,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     const float st_mul = tid < BM ? -1.f / p.scale : -1.f;  // threads 0..63 stage -LSE/scale, 64..127 stage -DELTA
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
+    int sld_row0 = 0;     // first row of the tile in flight
     unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * (L::P_SLOT / 4);
 
     // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
@@ -1013,6 +1011,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         auto gload = [&](int rep, int qt, int buf) {
             const int h = hkv * p.n_rep + rep;
             const int row0 = qt * BM;
+            sld_row0 = row0;
             const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
             const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
             const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
@@ -1043,17 +1042,14 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 // rows past the end: -LSE/scale = -inf makes P = 0 (they are masked as well)
                 if (MASK) x = sld_ok ? x : (tid < BM ? -INFINITY : 0.f);
                 st[tid] = x;
+            } else if (MASK && tid < 3 * BM) {   // positions of the tile's rows (third wave)
+                const int row = sld_row0 + tid - 2 * BM;
+                ((int *)st)[tid] = row >= p.Sq ? BWD_QPOS_NONE
+                                   : causal ? q_position(row, p.q_split, p.q_pos0[0], p.q_pos0[1]) : BWD_QPOS_ALL;
             }
         };
 
-        BwdMaskCtx mctx;
-        mctx.key_ok = key_ok;
-        mctx.causal = causal;
-        mctx.my_kpos = pos0 + my_key;
-        mctx.Sq = p.Sq;
-        mctx.q_split = p.q_split;
-        mctx.p0 = p.q_pos0[0];
-        mctx.p1 = p.q_pos0[1];
+        const int kpos = key_ok ? pos0 + my_key : BWD_KPOS_NONE;
         if (cnt == 0) return;
         int rep = 0, qt = 0;
         advance(rep, qt);
@@ -1081,7 +1077,6 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             bool more = true;
             auto p_step = [&](auto buf_tag) {
                 const int buf = buf_tag;
-                mctx.row_base = qt * BM;
                 more = advance(rep, qt);
                 const int nbuf = buf == L::NBUF - 1 ? 0 : buf + 1;
                 if (more) gload(rep, qt, nbuf);
@@ -1103,13 +1098,25 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                         sb[4 * g + e] = lb[e];
                     }
                 }
+                int qa[16], qb[16];   // positions of the rows (masked tiles only)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int *st_q = (const int *)st_s + 2 * BM;
+                    const i32x4 xa = MASK ? *(const i32x4 *)(st_q + 8 * g + 4 * hh) : i32x4{0, 0, 0, 0};
+                    const i32x4 xb = MASK ? *(const i32x4 *)(st_q + 32 + 8 * g + 4 * hh) : i32x4{0, 0, 0, 0};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        qa[4 * g + e] = xa[e];
+                        qb[4 * g + e] = xb[e];
+                    }
+                }
                 PackedTile ppa, ppb;
                 constexpr int NK = D / 16, ND = D / 32;
                 __builtin_amdgcn_s_setprio(1);
                 lds_gemm_chain<D>(Qs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, sa);
                 lds_gemm_chain<D>(Qs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, sb, [&](int kb) {
 #pragma unroll
-                    for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) ppa.u[j] = bwd_p_pair<MASK>(sa, j, 0, hh, c2, mctx);
+                    for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) ppa.u[j] = bwd_p_pair<MASK>(sa, j, c2, kpos, qa);
                 });
                 put_slot(slots, ppa);
                 bf16x8 pb[4];
@@ -1119,7 +1126,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
                 // runs, and the loop reads pb[2], pb[3] only after that; the first half reads pb[0], pb[1]
                 lds_tr_gemm<D, 2>(dOs, 0, lane, *(const bf16x8(*)[2]) & pb[0], acc, [&](int step) {
 #pragma unroll
-                    for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) ppb.u[j] = bwd_p_pair<MASK>(sb, j, 32, hh, c2, mctx);
+                    for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) ppb.u[j] = bwd_p_pair<MASK>(sb, j, c2, kpos, qb);
                 });
                 put_slot(slots + L::P_SLOT / 4, ppb);
                 pb[2] = operand_of(ppb, 0);
