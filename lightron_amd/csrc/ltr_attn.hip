@@ -363,6 +363,45 @@ __device__ __forceinline__ void lds_tr_gemm_at(const unsigned (&addr)[D / 32][2]
     }
 }
 
+// Epilogue helper: a wave turns its 32 x D result tile, held in MFMA accumulator layout (lane (row l32, half hh),
+// accumulator (db, 4 g + e) -> column 32 db + 8 g + 4 hh + e), into row-major order through a wave-private LDS area, so
+// that global memory is written (and, for accumulators, read) in runs of whole rows instead of 8-16 bytes per row
+// and instruction.  emit(row, col, v) receives 4 consecutive columns of one row; 32 / (D / 4) ... rows per step.
+template <int D>
+struct WaveStage {
+    static constexpr int ROW_BYTES = D * 4 + 16;          // padded rows: the 128-bit column writes hit every bank once
+    static constexpr int BYTES = 32 * ROW_BYTES + 128;    // + one float per row (per-row factor of the caller)
+};
+
+// Wave-uniform values pinned in scalar registers: kernel arguments used inside the epilogue loops are otherwise
+// re-read from the argument segment in every iteration (a scalar load and a wait each time).
+__device__ __forceinline__ int uniform32(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ long long uniform64(long long x) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)x), hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(x >> 32));
+    return (long long)(((unsigned long long)hi << 32) | lo);
+}
+
+template <int D, class Emit>
+__device__ __forceinline__ void wave_tile_rowmajor(unsigned char *stage, int lane, const f32x16 (&acc)[D / 32], float mul,
+                                                   Emit emit) {
+    const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int db = 0; db < D / 32; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = acc[db][4 * g + e] * mul;
+            *(f32x4 *)(stage + l32 * WaveStage<D>::ROW_BYTES + (32 * db + 8 * g + 4 * hh) * 4) = v;
+        }
+    constexpr int LPR = D / 4;                // lanes per row
+#pragma unroll
+    for (int it = 0; it < 32 * LPR / 64; it++) {
+        const int idx = it * 64 + lane, row = idx / LPR, c4 = idx % LPR;
+        emit(row, 4 * c4, *(const f32x4 *)(stage + row * WaveStage<D>::ROW_BYTES + c4 * 16));
+    }
+}
+
 // keys per K / V tile of the forward and dQ kernels
 template <int D>
 struct FwdTile {
@@ -638,38 +677,47 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             lse_new = mxl + logf(tot);
         }
     }
-    if (row_ok) {
-        if (hh == 0) *lse_p = lse_new;
-        const long long ooff = b * p.os[0] + (long long)my_row * p.os[1] + h * p.os[2];
+    if (row_ok && hh == 0) *lse_p = lse_new;
+    // O through the wave's LDS staging area (the tiles are no longer read: the last barrier is behind us)
+    unsigned char *stage = smem + w * WaveStage<D>::BYTES;
+    float *row_w_old = (float *)(stage + 32 * WaveStage<D>::ROW_BYTES);
+    if (hh == 0) row_w_old[l32] = w_old;
+    constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
+    const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + w * 32);
+    const bool merge = uniform32(p.flags & LTR_MERGE) != 0, o_f32 = uniform32(p.o_f32) != 0;
+    const long long os1 = uniform64(p.os[1]);
+    const long long off0 = uniform64(b * p.os[0] + h * p.os[2]) + (wave_row0 + lane / LPR) * os1 + 4 * (lane % LPR);
+    if (o_f32) {
+        float *op = (float *)p.o + off0;
+        wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
+            if (wave_row0 + row < Sq_u) {
+                if (merge) {
+                    const f32x4 old = *(const f32x4 *)op;
+                    const float wo = row_w_old[row];
 #pragma unroll
-        for (int db = 0; db < D / 32; db++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d = db * 32 + 8 * g + 4 * hh;
-                f32x4 val;
-#pragma unroll
-                for (int e = 0; e < 4; e++) val[e] = oacc[db][4 * g + e] * w_cur;
-                if (p.o_f32) {
-                    float *op = (float *)p.o + ooff + d;
-                    if (p.flags & LTR_MERGE) {
-                        f32x4 old = *(const f32x4 *)op;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) val[e] += old[e] * w_old;
-                    }
-                    *(f32x4 *)op = val;
-                } else {
-                    __bf16 *op = (__bf16 *)p.o + ooff + d;
-                    if (p.flags & LTR_MERGE) {
-                        bf16x4 old = *(const bf16x4 *)op;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) val[e] += (float)old[e] * w_old;
-                    }
-                    bf16x4 ob;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) ob[e] = (__bf16)val[e];
-                    *(bf16x4 *)op = ob;
+                    for (int e = 0; e < 4; e++) val[e] += old[e] * wo;
                 }
+                *(f32x4 *)op = val;
             }
+            op += ROWS_PER_IT * os1;
+        });
+    } else {
+        __bf16 *op = (__bf16 *)p.o + off0;
+        wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
+            if (wave_row0 + row < Sq_u) {
+                if (merge) {
+                    const bf16x4 old = *(const bf16x4 *)op;
+                    const float wo = row_w_old[row];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) val[e] += (float)old[e] * wo;
+                }
+                bf16x4 ob;
+#pragma unroll
+                for (int e = 0; e < 4; e++) ob[e] = (__bf16)val[e];
+                *(bf16x4 *)op = ob;
+            }
+            op += ROWS_PER_IT * os1;
+        });
     }
 }
 
@@ -1704,7 +1752,9 @@ int check_device() {
 
 // kernels that need more than 64 KB of dynamic LDS must opt in once per process
 template <int D>
-constexpr int fwd_lds_bytes() { return 2 * 2 * FwdTile<D>::BN * D * 2; }
+constexpr int fwd_lds_bytes() {   // the K / V tile buffers, reused by the epilogue's staging areas (one per wave)
+    return 2 * 2 * FwdTile<D>::BN * D * 2 > 8 * WaveStage<D>::BYTES ? 2 * 2 * FwdTile<D>::BN * D * 2 : 8 * WaveStage<D>::BYTES;
+}
 template <int D>
 constexpr int dq_lds_bytes() { return 2 * 2 * FwdTile<D>::BN * D * 2; }
 
