@@ -892,6 +892,7 @@ struct BwdLds {
     static constexpr int MAX_QTILES = 4096;                              // Sq <= 262144 per launch
     static constexpr int LIST_OFF = P_OFF + 4 * 4 * P_SLOT;              // 4 slices x 2 parities x 2 sub-tiles of P slots
     static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;     // two tile lists (ushort) + counts
+    static_assert(TOTAL >= 8 * WaveStage<D>::BYTES, "the epilogue's staging areas reuse this memory");
 };
 
 // Masked tiles: the visibility of (row, key) is kpos <= qpos[row], with the rows' positions staged in LDS beside LSE and
@@ -1280,21 +1281,32 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     run_pass(std::false_type{});
     run_pass(std::true_type{});
 
-    // dV^T (P wave) / dK^T (dS wave) tile: lane (key l32 of the slice, half hh), register r -> d = 32*db + 8*(r/4) + 4hh + r%4
-    if (key_ok) {
-        float *gp = p_role ? p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2]
-                           : p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2];
-        const float mul = p_role ? 1.f : p.scale;
+    // dV^T (P wave) / dK^T (dS wave) tile of the wave's 32 keys: added to the fp32 accumulators in whole rows, through the
+    // wave's LDS staging area (every wave is past the last barrier: tiles, slots and lists are no longer read)
+    {
+        constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
+        const long long stride = uniform64(p_role ? p.dvs[1] : p.dks[1]);
+        const int key_base = uniform32(key0 + slice * 32), sk_u = uniform32(sk);
+        float *gp = (p_role ? p.chunk[c].dv + b * p.dvs[0] + hkv * p.dvs[2] : p.chunk[c].dk + b * p.dks[0] + hkv * p.dks[2]) +
+                    (key_base + lane / LPR) * stride + 4 * (lane % LPR);
+        // all reads of the accumulator first (independent loads in flight together), then the adds and the writes
+        constexpr int NIT = 32 / ROWS_PER_IT;
+        f32x4 old[NIT];
 #pragma unroll
-        for (int db = 0; db < D / 32; db++)
+        for (int it = 0; it < NIT; it++) {
+            old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (key_base + it * ROWS_PER_IT + lane / LPR < sk_u) old[it] = *(const f32x4 *)(gp + it * ROWS_PER_IT * stride);
+        }
+        int it = 0;
+        wave_tile_rowmajor<D>(smem + w * WaveStage<D>::BYTES, lane, acc, p_role ? 1.f : p.scale, [&](int row, int, f32x4 val) {
+            if (key_base + row < sk_u) {
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d = db * 32 + 8 * g + 4 * hh;
-                f32x4 old = *(const f32x4 *)(gp + d);
-#pragma unroll
-                for (int e = 0; e < 4; e++) old[e] += acc[db][4 * g + e] * mul;
-                *(f32x4 *)(gp + d) = old;
+                for (int e = 0; e < 4; e++) val[e] += old[it][e];
+                *(f32x4 *)gp = val;
             }
+            gp += ROWS_PER_IT * stride;
+            it++;
+        });
     }
 }
 
@@ -1505,31 +1517,43 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
         have = have_next;
     }
 
-    if (row_ok) {
-        const long long off = b * p.dqs[0] + (long long)my_row * p.dqs[1] + h * p.dqs[2];
-        if (p.flags & LTR_DQ_BF16) {   // this call saw every key of these rows: store the result, no accumulator
-            __bf16 *dqp = (__bf16 *)p.dq + off;
-#pragma unroll
-            for (int db = 0; db < D / 32; db++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
+    // dQ in whole rows through the wave's LDS staging area (the tiles are no longer read: the last barrier is behind us)
+    {
+        constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
+        unsigned char *stage = smem + w * WaveStage<D>::BYTES;
+        const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + w * 32);
+        const long long dqs1 = uniform64(p.dqs[1]);
+        const long long off0 = uniform64(b * p.dqs[0] + h * p.dqs[2]) + (wave_row0 + lane / LPR) * dqs1 + 4 * (lane % LPR);
+        if (uniform32(p.flags & LTR_DQ_BF16)) {   // this call saw every key of these rows: store the result, no accumulator
+            __bf16 *dqp = (__bf16 *)p.dq + off0;
+            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int, f32x4 val) {
+                if (wave_row0 + row < Sq_u) {
                     bf16x4 y;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) y[e] = (__bf16)(dqacc[db][4 * g + e] * p.scale);
-                    *(bf16x4 *)(dqp + db * 32 + 8 * g + 4 * hh) = y;
+                    for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
+                    *(bf16x4 *)dqp = y;
                 }
+                dqp += ROWS_PER_IT * dqs1;
+            });
         } else {
-            float *dqp = (float *)p.dq + off;
+            float *dqp = (float *)p.dq + off0;
+            constexpr int NIT = 32 / ROWS_PER_IT;
+            f32x4 old[NIT];   // all reads of the accumulator first, then the adds and the writes
 #pragma unroll
-            for (int db = 0; db < D / 32; db++)
+            for (int it = 0; it < NIT; it++) {
+                old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (wave_row0 + it * ROWS_PER_IT + lane / LPR < Sq_u) old[it] = *(const f32x4 *)(dqp + it * ROWS_PER_IT * dqs1);
+            }
+            int it = 0;
+            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int, f32x4 val) {
+                if (wave_row0 + row < Sq_u) {
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int d = db * 32 + 8 * g + 4 * hh;
-                    f32x4 old = *(const f32x4 *)(dqp + d);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) old[e] += dqacc[db][4 * g + e] * p.scale;
-                    *(f32x4 *)(dqp + d) = old;
+                    for (int e = 0; e < 4; e++) val[e] += old[it][e];
+                    *(f32x4 *)dqp = val;
                 }
+                dqp += ROWS_PER_IT * dqs1;
+                it++;
+            });
         }
     }
 }
@@ -1756,7 +1780,7 @@ constexpr int fwd_lds_bytes() {   // the K / V tile buffers, reused by the epilo
     return 2 * 2 * FwdTile<D>::BN * D * 2 > 8 * WaveStage<D>::BYTES ? 2 * 2 * FwdTile<D>::BN * D * 2 : 8 * WaveStage<D>::BYTES;
 }
 template <int D>
-constexpr int dq_lds_bytes() { return 2 * 2 * FwdTile<D>::BN * D * 2; }
+constexpr int dq_lds_bytes() { return fwd_lds_bytes<D>(); }   // same tile buffers and staging areas as the forward
 
 int enable_large_lds() {
     static int done = 0;  // 0 not yet, 1 ok, -1 failed
