@@ -687,29 +687,45 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     const bool merge = uniform32(p.flags & LTR_MERGE) != 0, o_f32 = uniform32(p.o_f32) != 0;
     const long long os1 = uniform64(p.os[1]);
     const long long off0 = uniform64(b * p.os[0] + h * p.os[2]) + (wave_row0 + lane / LPR) * os1 + 4 * (lane % LPR);
+    // merging: all reads of the earlier partial result first (independent loads in flight together), then the writes
+    constexpr int NIT = 32 / ROWS_PER_IT;
+    f32x4 old[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (merge && wave_row0 + it * ROWS_PER_IT + lane / LPR < Sq_u) {
+            if (o_f32) {
+                old[it] = *(const f32x4 *)((const float *)p.o + off0 + it * ROWS_PER_IT * os1);
+            } else {
+                const bf16x4 x = *(const bf16x4 *)((const __bf16 *)p.o + off0 + it * ROWS_PER_IT * os1);
+#pragma unroll
+                for (int e = 0; e < 4; e++) old[it][e] = (float)x[e];
+            }
+        }
+    }
+    int it = 0;
     if (o_f32) {
         float *op = (float *)p.o + off0;
         wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
             if (wave_row0 + row < Sq_u) {
                 if (merge) {
-                    const f32x4 old = *(const f32x4 *)op;
                     const float wo = row_w_old[row];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) val[e] += old[e] * wo;
+                    for (int e = 0; e < 4; e++) val[e] += old[it][e] * wo;
                 }
                 *(f32x4 *)op = val;
             }
             op += ROWS_PER_IT * os1;
+            it++;
         });
     } else {
         __bf16 *op = (__bf16 *)p.o + off0;
         wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
             if (wave_row0 + row < Sq_u) {
                 if (merge) {
-                    const bf16x4 old = *(const bf16x4 *)op;
                     const float wo = row_w_old[row];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) val[e] += (float)old[e] * wo;
+                    for (int e = 0; e < 4; e++) val[e] += old[it][e] * wo;
                 }
                 bf16x4 ob;
 #pragma unroll
@@ -717,6 +733,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
                 *(bf16x4 *)op = ob;
             }
             op += ROWS_PER_IT * os1;
+            it++;
         });
     }
 }
