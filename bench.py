@@ -201,8 +201,12 @@ def main():
         # every rank's call holds all KV chunks its queries see, so the dQ kernel writes bf16 dQ itself (LTR_DQ_BF16)
         dq_out = torch.empty(q_all.shape, dtype=torch.bfloat16, device=dev)
         delta_ws = torch.empty(B, Hq, sl, dtype=torch.float32, device=dev)
-        dk_acc = torch.empty(k_all.shape, dtype=torch.float32, device=dev)
-        dv_acc = torch.empty(v_all.shape, dtype=torch.float32, device=dev)
+        # dK / dV: fp32 accumulators summed over the rank shares and cast at the end; when the workload is ONE share that
+        # holds the whole sequence (config 5) the kernel writes the bf16 results itself (LTR_DKDV_BF16)
+        dkdv_direct = W == 1 and len(cfg["ranks"]) == 1
+        acc_dtype = torch.bfloat16 if dkdv_direct else torch.float32
+        dk_acc = torch.empty(k_all.shape, dtype=acc_dtype, device=dev)
+        dv_acc = torch.empty(v_all.shape, dtype=acc_dtype, device=dev)
 
     def acc_views(r, acc):
         out = []
@@ -227,7 +231,7 @@ def main():
         return r
 
     def step(timed):
-        if bwd:
+        if bwd and not dkdv_direct:
             dk_acc.zero_(); dv_acc.zero_()
         for r in cfg["ranks"]:
             ks, vs, pos, qp, qsplit = tables[r]
@@ -243,7 +247,7 @@ def main():
                 timed_call("dkdv", timed, lambda: la.attn_bwd_accumulate(
                     q_all[r], do_all[r], lse_all[r], delta_ws, ks, vs, pos, dq_out[r], dks, dvs, qp, qsplit, causal,
                     do_dq=False))
-        if bwd:
+        if bwd and not dkdv_direct:
             la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
 
     for _ in range(args.warmup):

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 2
+#define LTR_ABI_VERSION 3
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -49,6 +49,7 @@ extern "C" {
 #define LTR_NO_DKDV 8u  /* backward: skip the dK/dV kernel (chunk[].dk/dv may be NULL) */
 #define LTR_DQ_BF16 16u /* backward: dq is a bf16 tensor that RECEIVES dQ of this call (no accumulation) */
 #define LTR_DELTA_FROM_O 32u /* backward: delta is computed from o by the dQ kernel (and written to delta) */
+#define LTR_DKDV_BF16 64u /* backward: chunk[c].dk / dv are bf16 tensors that RECEIVE dK / dV of this call (no accumulation) */
 
 /* error codes */
 #define LTR_OK 0
@@ -61,7 +62,7 @@ extern "C" {
 typedef struct ltr_kv_chunk {
     const void *k; /* [B, sk, Hkv, D] by kv strides */
     const void *v;
-    void *dk;      /* fp32 accumulators, same logical shape, by dkv strides (backward only) */
+    void *dk;      /* fp32 accumulators (bf16 results with LTR_DKDV_BF16), same logical shape, by dk/dv strides (backward only) */
     void *dv;
     int64_t sk;    /* keys in this chunk */
     int64_t pos0;  /* global position of its first key */
@@ -139,7 +140,11 @@ int ltr_attn_bwd_delta(const ltr_attn_delta_args *args, void *stream);
  * elements): no fp32 accumulator, no zero-fill, no final cast.  LTR_DELTA_FROM_O: delta is
  * an OUTPUT workspace; the dQ kernel computes DELTA = rowsum(dO * O) of its rows from o
  * (bf16, o_stride) and stores it, and the dK/dV kernel, enqueued after it, reads it: no
- * separate ltr_attn_bwd_delta launch.  Not combinable with LTR_NO_DQ.
+ * separate ltr_attn_bwd_delta launch.  Not combinable with LTR_NO_DQ.  LTR_DKDV_BF16: when q holds
+ * every query row that sees the keys of this call's chunks (one rank's own backward, not a ring step whose dK/dV
+ * go on to other ranks), dK / dV of those chunks are complete after the call: chunk[c].dk / dv may then be the
+ * bf16 results themselves (written for every key, zeros where no query sees it; dk/dv strides in bf16 elements):
+ * no fp32 accumulators, no zero-fill, no final cast.  bf16 only.
  */
 typedef struct ltr_attn_bwd_args {
     const void *q;
@@ -159,9 +164,9 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;
-    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 */
     int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: scalar fp32 kernels for the 1e-4 parity cases;
-                             LTR_DQ_BF16 and LTR_DELTA_FROM_O are bf16 only and return LTR_EUNSUP with it) */
+                             LTR_DQ_BF16, LTR_DELTA_FROM_O and LTR_DKDV_BF16 are bf16 only and return LTR_EUNSUP with it) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
     const void *o;        /* forward output, bf16, only read with LTR_DELTA_FROM_O */

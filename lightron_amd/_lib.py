@@ -7,10 +7,10 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
 
-LTR_ABI_VERSION = 2
+LTR_ABI_VERSION = 3
 LTR_MAX_CHUNKS = 32
 LTR_BF16, LTR_F32 = 0, 1
-LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O = 1, 2, 4, 8, 16, 32
+LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LTR_DKDV_BF16 = 1, 2, 4, 8, 16, 32, 64
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_abi_version", "ltr_strerror")

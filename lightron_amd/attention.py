@@ -136,7 +136,9 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
     queries can see and fit one launch (at most 32 chunks).  With o (the bf16 forward output) given, delta is a
     workspace: the dQ kernel of the first launch computes rowsum(dO * O) into it (LTR_DELTA_FROM_O) and no
-    attn_delta call is needed; this needs do_dq."""
+    attn_delta call is needed; this needs do_dq.  dk_accs / dv_accs may be bf16 tensors as well: they then RECEIVE
+    dK / dV (LTR_DKDV_BF16; every key is written), which is only right when q holds every query row that sees
+    these keys - one rank's own backward, not a ring step whose dK/dV are summed over ranks."""
     lib = _lib.load()
     _req(q, "q")
     _req(do, "dO")
@@ -147,12 +149,19 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     dq_direct = dq_acc.dtype == torch.bfloat16
     if dq_direct and do_dq and len(ks) > _lib.LTR_MAX_CHUNKS:
         raise RuntimeError("a bf16 dQ output needs all KV chunks in one launch (at most %d)" % _lib.LTR_MAX_CHUNKS)
-    for t in ([] if dq_direct else [dq_acc]) + list(dk_accs) + list(dv_accs):
+    dkdv_direct = dk_accs[0].dtype == torch.bfloat16
+    for t in list(dk_accs) + list(dv_accs):
+        if t.dtype != dk_accs[0].dtype:
+            raise RuntimeError("dK / dV tensors must share one dtype (fp32 accumulators or bf16 results)")
+    for t in ([] if dq_direct else [dq_acc]) + ([] if dkdv_direct else list(dk_accs) + list(dv_accs)):
         _req(t, "accumulator")
         if t.dtype != torch.float32:
             raise RuntimeError("gradient accumulators must be fp32")
     if dq_direct:
         _req(dq_acc, "dQ")
+    if dkdv_direct:
+        for t in list(dk_accs) + list(dv_accs):
+            _req(t, "dK / dV")
     a = _lib.BwdArgs()
     a.q, a.d_o, a.lse, a.delta, a.dq = q.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(), dq_acc.data_ptr()
     a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, ks[0].shape[2], D, Sq
@@ -162,7 +171,8 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
     a.flags = ((_lib.LTR_CAUSAL if causal else 0) | (0 if do_dq else _lib.LTR_NO_DQ)
-               | (0 if do_dkdv else _lib.LTR_NO_DKDV) | (_lib.LTR_DQ_BF16 if dq_direct else 0))
+               | (0 if do_dkdv else _lib.LTR_NO_DKDV) | (_lib.LTR_DQ_BF16 if dq_direct else 0)
+               | (_lib.LTR_DKDV_BF16 if dkdv_direct else 0))
     a.io_dtype = _DT[q.dtype]
     if o is not None:
         if not do_dq:
@@ -237,21 +247,24 @@ class BlockAttentionFunction(torch.autograd.Function):
         direct = n_chunks <= _lib.LTR_MAX_CHUNKS and not f32
         dq_acc = (torch.empty(q.shape, dtype=torch.bfloat16, device=q.device) if direct
                   else torch.zeros(q.shape, dtype=torch.float32, device=q.device))
-        # one fp32 buffer per gradient, sliced along the sequence: every chunk's accumulator has the same strides
+        # one buffer per gradient, sliced along the sequence: every chunk's slice has the same strides.  This node's
+        # q holds every query that sees these keys inside this node (autograd sums over nodes by itself), so for bf16
+        # the kernels write dK / dV directly: no fp32 accumulators, no zero-fill, no cast.
         lens = [k.shape[1] for k in ks]
         shape = (ks[0].shape[0], sum(lens), ks[0].shape[2], ks[0].shape[3])
-        dk_buf = torch.zeros(shape, dtype=torch.float32, device=q.device)
-        dv_buf = torch.zeros(shape, dtype=torch.float32, device=q.device)
+        if f32:
+            dk_buf = torch.zeros(shape, dtype=torch.float32, device=q.device)
+            dv_buf = torch.zeros(shape, dtype=torch.float32, device=q.device)
+        else:
+            dk_buf = torch.empty(shape, dtype=torch.bfloat16, device=q.device)
+            dv_buf = torch.empty(shape, dtype=torch.bfloat16, device=q.device)
         offs = [sum(lens[:i]) for i in range(len(lens))]
         dk_accs = [dk_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         dv_accs = [dv_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale,
                             o=o if fuse else None)
-        if f32:   # the fp32 kernels accumulate into the gradients themselves
-            dq, dk16, dv16 = dq_acc, dk_buf, dv_buf
-        else:
-            dq = dq_acc if direct else cast_to_bf16(dq_acc)
-            dk16, dv16 = cast_to_bf16(dk_buf), cast_to_bf16(dv_buf)
+        dq = dq_acc if (direct or f32) else cast_to_bf16(dq_acc)
+        dk16, dv16 = dk_buf, dv_buf
         dks = [dk16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         dvs = [dv16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         return (dq, None, None, None, None, None, None, None, None, *dks, *dvs)

@@ -982,7 +982,14 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     if (causal) {   // no query of this launch sees the block (a later chunk of the ring): nothing to add, nothing to load
         int q_lo, q_hi;
         q_pos_range(0, (int)p.Sq - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], q_lo, q_hi);
-        if (q_hi < tile_kpos_lo) return;
+        if (q_hi < tile_kpos_lo) {
+            if ((p.flags & LTR_DKDV_BF16) && key_ok) {   // results, not accumulators: these keys get zeros
+                __bf16 *gz = p_role ? (__bf16 *)p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2]
+                                    : (__bf16 *)p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2];
+                for (int d = 8 * hh; d < D; d += 16) *(uint4 *)(gz + d) = make_uint4(0, 0, 0, 0);
+            }
+            return;
+        }
     }
 
     // resident B operand: K rows for a P wave, V rows for a dS wave; lane (key l32, half hh) holds
@@ -1304,8 +1311,22 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
         const long long stride = uniform64(p_role ? p.dvs[1] : p.dks[1]);
         const int key_base = uniform32(key0 + slice * 32), sk_u = uniform32(sk);
-        float *gp = (p_role ? p.chunk[c].dv + b * p.dvs[0] + hkv * p.dvs[2] : p.chunk[c].dk + b * p.dks[0] + hkv * p.dks[2]) +
-                    (key_base + lane / LPR) * stride + 4 * (lane % LPR);
+        const long long goff = (p_role ? b * p.dvs[0] + hkv * p.dvs[2] : b * p.dks[0] + hkv * p.dks[2]) +
+                               (key_base + lane / LPR) * stride + 4 * (lane % LPR);
+        if (uniform32(p.flags & LTR_DKDV_BF16)) {   // every query that sees these keys was in this launch: store the result
+            __bf16 *gb = (__bf16 *)(p_role ? p.chunk[c].dv : p.chunk[c].dk) + goff;
+            wave_tile_rowmajor<D>(smem + w * WaveStage<D>::BYTES, lane, acc, p_role ? 1.f : p.scale, [&](int row, int, f32x4 val) {
+                if (key_base + row < sk_u) {
+                    bf16x4 y;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
+                    *(bf16x4 *)gb = y;
+                }
+                gb += ROWS_PER_IT * stride;
+            });
+            return;
+        }
+        float *gp = (p_role ? p.chunk[c].dv : p.chunk[c].dk) + goff;
         // all reads of the accumulator first (independent loads in flight together), then the adds and the writes
         constexpr int NIT = 32 / ROWS_PER_IT;
         f32x4 old[NIT];
@@ -1954,19 +1975,20 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O)) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16)) return LTR_EINVAL;
     const bool fused_delta = a->flags & LTR_DELTA_FROM_O;
     if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     const bool f32 = a->io_dtype == LTR_F32;
-    if (f32 && (a->flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O))) return LTR_EUNSUP;   // bf16 conveniences only
+    if (f32 && (a->flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16))) return LTR_EUNSUP;   // bf16 conveniences only
+    const int gb = (a->flags & LTR_DKDV_BF16) ? 2 : 4;   // bytes per dK / dV element
     const int eb = f32 ? 4 : 2;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
     if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
     if (!aligned16(a->q) || !aligned16(a->d_o) || (do_dq && !aligned16(a->dq))) return LTR_EALIGN;
     if (!strides_ok(a->q_stride, eb) || !strides_ok(a->do_stride, eb) || !strides_ok(a->k_stride, eb) ||
-        !strides_ok(a->v_stride, eb) || !strides_ok(a->dk_stride, 4) || !strides_ok(a->dv_stride, 4))
+        !strides_ok(a->v_stride, eb) || !strides_ok(a->dk_stride, gb) || !strides_ok(a->dv_stride, gb))
         return LTR_EALIGN;
     for (int i = 0; i < 3; i++)
         if (a->dq_stride[i] < 0) return LTR_EINVAL;

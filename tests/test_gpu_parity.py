@@ -464,6 +464,35 @@ def test_dq_written_as_bf16_equals_accumulate_then_cast(ltr):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D,Hq,Hkv,Sq,q0,causal", [(128, 4, 2, 300, 0, True), (64, 2, 2, 100, 150, True),
+                                                   (128, 2, 1, 77, 40, False), (64, 4, 1, 256, 1000, True)])
+def test_dkdv_written_as_bf16_equals_accumulate_then_cast(ltr, D, Hq, Hkv, Sq, q0, causal):
+    """LTR_DKDV_BF16 (dk / dv receive the bf16 results of a call whose q holds every query that sees the keys) against
+    the fp32 accumulator path followed by the cast: the same value is rounded once in both, so the bits agree; keys
+    that no query sees (whole 128-key blocks of them included) are written as zeros."""
+    g = torch.Generator().manual_seed(21)
+    B, sks, pos0 = 2, [200, 130, 400], [0, 200, 330]
+    q, do = (torch.randn(B, Sq, Hq, D, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+    kf, vf = (torch.randn(B, sum(sks), Hkv, D, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+    offs = [0, 200, 330]
+    cut = lambda t: [t[:, o_:o_ + n_] for o_, n_ in zip(offs, sks)]
+    ks, vs = cut(kf), cut(vf)
+    o, lse = ltr.attn_fwd(q, ks, vs, pos0, q0, None, causal)
+    delta = ltr.attn_delta(o, do)
+    dq = torch.empty_like(q)
+    dkf, dvf = (torch.zeros(kf.shape, dtype=torch.float32, device="cuda") for _ in range(2))
+    ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, dq, cut(dkf), cut(dvf), q0, None, causal, do_dq=False)
+    dkb, dvb = (torch.full(kf.shape, float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(2))
+    ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, dq, cut(dkb), cut(dvb), q0, None, causal, do_dq=False)
+    assert torch.equal(dkb, ltr.cast_to_bf16(dkf))
+    assert torch.equal(dvb, ltr.cast_to_bf16(dvf))
+    if causal and q0 + Sq <= 330:
+        assert dkb[:, 330:].abs().max() == 0 and dvb[:, 330:].abs().max() == 0   # keys after every query
+    with pytest.raises(RuntimeError):   # mixed dtypes
+        ltr.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos0, dq, cut(dkb), cut(dvf), q0, None, causal, do_dq=False)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("case", ["huge_positive", "huge_negative", "mixed_rows", "growing"])
 def test_extreme_logits(ltr, case):
     """Scores far outside the range where exp2 of (score - fixed reference) is representable: the forward's
