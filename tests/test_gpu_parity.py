@@ -221,10 +221,11 @@ def test_fp32_backward_random_shapes(ltr, seed):
     for name, a, b in (("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
         assert a.dtype == torch.float32
         assert torch.isfinite(a).all(), name
-        if b.abs().max() > 0:
+        # (a single visible key gives dS = P (dP - DELTA) = 0 exactly: only an absolute bound makes sense there)
+        if b.abs().max() > 1e-3:
             assert _rel(a.cpu(), b) < F32_TOL, (name, _rel(a.cpu(), b))
         else:
-            assert a.abs().max() == 0, name
+            assert (a.cpu().double() - b).abs().max() < F32_TOL, name
 
 
 def test_ragged_bwd(ltr):
