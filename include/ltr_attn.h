@@ -9,7 +9,10 @@
  * synchronising.  The library never allocates, frees or keeps a pointer after the
  * call returns; all buffers, including fp32 gradient accumulators, belong to the
  * caller.  Return value: 0 on success, a negative LTR_E* code otherwise (nothing is
- * enqueued on error).  Re-entrant; no mutable global state.
+ * enqueued on error).  Re-entrant and safe to call from several host threads: the only
+ * mutable global state is a small per-device record of facts found out on the first call
+ * on each device (architecture check, large-LDS opt-in), kept in atomics and read-only
+ * afterwards.
  *
  * Tensor layout: element strides (in elements, not bytes) are given for the batch,
  * sequence and head dimensions; the head dimension D is contiguous.  This serves

@@ -36,6 +36,7 @@
 #include <stdint.h>
 #include <math.h>
 #include <type_traits>
+#include <atomic>
 #include "ltr_attn.h"
 
 namespace {
@@ -190,7 +191,7 @@ __device__ __forceinline__ unsigned lds_address(const void *shared_object) {
 
 __device__ __forceinline__ void global_to_lds_b128(const void *gptr, unsigned lds_byte_addr_uniform) {
     const unsigned lds_addr = __builtin_amdgcn_readfirstlane(lds_byte_addr_uniform);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
 
 // End of a tile: wait for every outstanding tile transfer and LDS access of this wave, then the block
@@ -1799,20 +1800,36 @@ __global__ __launch_bounds__(64) void bwd_dkdv_f32_kernel(const BwdParams p) {
 // ------------------------------------------------------------------------------ host side
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-int check_device() {
-    // gfx950 only; the answer is cached per process (read-only after first use)
-    static int cached = 0;  // 0 unknown, 1 ok, -1 bad
-    if (cached == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_EDEVICE;
-        const char *a = prop.gcnArchName;
-        cached = (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') ? 1 : -1;
-    }
-    return cached == 1 ? LTR_OK : LTR_EDEVICE;
+// Per-device facts, found out on the first call on each device and read-only afterwards.  The fields are atomics: two host
+// threads that make their first call at the same time both do the (idempotent) work and store the same answer.  A failed
+// query or opt-in is not remembered: the next call tries again.
+constexpr int LTR_MAX_DEVICES = 64;
+struct DeviceState {
+    std::atomic<int> arch{0};          // 0 unknown, 1 gfx950, -1 something else
+    std::atomic<int> large_lds{0};     // 1: the kernels of this device may use more than 64 KB of dynamic LDS
+};
+DeviceState g_dev[LTR_MAX_DEVICES];
+
+int current_device(int *dev) {
+    if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= LTR_MAX_DEVICES) return LTR_EDEVICE;
+    return LTR_OK;
 }
 
-// kernels that need more than 64 KB of dynamic LDS must opt in once per process
+int check_device() {   // gfx950 only
+    int dev = 0;
+    if (current_device(&dev)) return LTR_EDEVICE;
+    int arch = g_dev[dev].arch.load(std::memory_order_acquire);
+    if (arch == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_EDEVICE;
+        const char *a = prop.gcnArchName;
+        arch = (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') ? 1 : -1;
+        g_dev[dev].arch.store(arch, std::memory_order_release);
+    }
+    return arch == 1 ? LTR_OK : LTR_EDEVICE;
+}
+
+// kernels that need more than 64 KB of dynamic LDS must opt in once per device
 template <int D>
 constexpr int fwd_lds_bytes() {   // the K / V tile buffers, reused by the epilogue's staging areas (one per wave)
     return 2 * 2 * FwdTile<D>::BN * D * 2 > 8 * WaveStage<D>::BYTES ? 2 * 2 * FwdTile<D>::BN * D * 2 : 8 * WaveStage<D>::BYTES;
@@ -1821,23 +1838,27 @@ template <int D>
 constexpr int dq_lds_bytes() { return fwd_lds_bytes<D>(); }   // same tile buffers and staging areas as the forward
 
 int enable_large_lds() {
-    static int done = 0;  // 0 not yet, 1 ok, -1 failed
-    if (done == 0) {
-        bool ok = hipFuncSetAttribute((const void *)bwd_dkdv_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      BwdLds<128>::TOTAL) == hipSuccess &&
-                  hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      BwdLds<64>::TOTAL) == hipSuccess &&
-                  hipFuncSetAttribute((const void *)fwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      fwd_lds_bytes<128>()) == hipSuccess &&
-                  hipFuncSetAttribute((const void *)fwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      fwd_lds_bytes<64>()) == hipSuccess &&
-                  hipFuncSetAttribute((const void *)bwd_dq_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      dq_lds_bytes<128>()) == hipSuccess &&
-                  hipFuncSetAttribute((const void *)bwd_dq_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      dq_lds_bytes<64>()) == hipSuccess;
-        done = ok ? 1 : -1;
+    int dev = 0;
+    if (current_device(&dev)) return LTR_EDEVICE;
+    if (g_dev[dev].large_lds.load(std::memory_order_acquire) == 1) return LTR_OK;
+    bool ok = hipFuncSetAttribute((const void *)bwd_dkdv_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  BwdLds<128>::TOTAL) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  BwdLds<64>::TOTAL) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  fwd_lds_bytes<128>()) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  fwd_lds_bytes<64>()) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  dq_lds_bytes<128>()) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  dq_lds_bytes<64>()) == hipSuccess;
+    if (!ok) {
+        (void)hipGetLastError();
+        return LTR_ELAUNCH;
     }
-    return done == 1 ? LTR_OK : LTR_ELAUNCH;
+    g_dev[dev].large_lds.store(1, std::memory_order_release);
+    return LTR_OK;
 }
 
 bool strides_ok(const int64_t *s, int elem_bytes) {
@@ -1969,20 +1990,22 @@ extern "C" int ltr_attn_bwd_delta(const ltr_attn_delta_args *a, void *stream) {
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
 
-extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
-    if (!a || !a->q || !a->d_o || !a->lse || !a->delta) return LTR_EINVAL;
-    const bool do_dq = !(a->flags & LTR_NO_DQ), do_dkdv = !(a->flags & LTR_NO_DKDV);
+namespace {
+int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, void *stream) {
+    float *delta = a->delta;
+    if (!a->q || !a->d_o || !a->lse || !delta) return LTR_EINVAL;
+    const bool do_dq = !(flags & LTR_NO_DQ), do_dkdv = !(flags & LTR_NO_DKDV);
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16)) return LTR_EINVAL;
-    const bool fused_delta = a->flags & LTR_DELTA_FROM_O;
+    if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16)) return LTR_EINVAL;
+    const bool fused_delta = flags & LTR_DELTA_FROM_O;
     if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     const bool f32 = a->io_dtype == LTR_F32;
-    if (f32 && (a->flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16))) return LTR_EUNSUP;   // bf16 conveniences only
-    const int gb = (a->flags & LTR_DKDV_BF16) ? 2 : 4;   // bytes per dK / dV element
+    if (f32 && (flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16))) return LTR_EUNSUP;   // bf16 conveniences only
+    const int gb = (flags & LTR_DKDV_BF16) ? 2 : 4;   // bytes per dK / dV element
     const int eb = f32 ? 4 : 2;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
     if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
@@ -1992,7 +2015,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
         return LTR_EALIGN;
     for (int i = 0; i < 3; i++)
         if (a->dq_stride[i] < 0) return LTR_EINVAL;
-    if (do_dq && !strides_ok(a->dq_stride, (a->flags & LTR_DQ_BF16) ? 2 : 4)) return LTR_EALIGN;
+    if (do_dq && !strides_ok(a->dq_stride, (flags & LTR_DQ_BF16) ? 2 : 4)) return LTR_EALIGN;
     if (fused_delta && (!aligned16(a->o) || !strides_ok(a->o_stride, 2))) return LTR_EALIGN;
     if (fused_delta && (a->Sq + 64) * a->o_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     if ((a->Sq + 63) / 64 > BwdLds<128>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
@@ -2019,7 +2042,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     p.q = a->q;
     p.d_o = a->d_o;
     p.lse = a->lse;
-    p.delta = a->delta;
+    p.delta = delta;
     p.o = a->o;
     for (int i = 0; i < 3; i++) p.os_[i] = fused_delta ? a->o_stride[i] : 0;
     p.dq = a->dq;
@@ -2042,7 +2065,7 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     p.q_pos0[1] = (int)a->q_pos0[1];
     p.q_split = (int)a->q_split;
     p.scale = a->scale;
-    p.flags = a->flags;
+    p.flags = flags;
     p.n_chunks = a->n_chunks;
     p.tiles_total = (int)tiles;
     const long long nblk = tiles * p.B * p.Hkv;
@@ -2081,6 +2104,12 @@ extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
         if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+}
+}  // namespace
+
+extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
+    if (!a) return LTR_EINVAL;
+    return bwd_launch(a, a->flags, stream);
 }
 
 extern "C" int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream) {

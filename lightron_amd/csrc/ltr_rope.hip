@@ -2,6 +2,7 @@
 // apply_rotary_emb (layers/layers.py:44-70) - adjacent pairs, fp32 complex multiply, cast back - without the
 // fp32 / complex temporaries that the torch formulation writes to HBM.  Bound: HBM (2 x element size per element).
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 #include "ltr_attn.h"
 
@@ -83,16 +84,22 @@ __global__ __launch_bounds__(256) void rope_kernel(const RopeParams p) {
     }
 }
 
+// gfx950 only.  The answer is kept per device in an atomic (two host threads making their first call together both do
+// the query and store the same value); a failed query is not remembered.
 bool on_gfx950() {
-    static int cached = 0;  // 0 unknown, 1 yes, -1 no (read-only after the first call)
-    if (cached == 0) {
-        int dev = 0;
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<int> arch[MAX_DEVICES];   // 0 unknown, 1 yes, -1 no
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return false;
+    int known = arch[dev].load(std::memory_order_acquire);
+    if (known == 0) {
         hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
         const char *a = prop.gcnArchName;
-        cached = (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') ? 1 : -1;
+        known = (a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0') ? 1 : -1;
+        arch[dev].store(known, std::memory_order_release);
     }
-    return cached == 1;
+    return known == 1;
 }
 
 }  // namespace
