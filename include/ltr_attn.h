@@ -8,11 +8,12 @@
  * as void*; NULL = the default stream) of the CURRENT device and returns without
  * synchronising.  The library never allocates, frees or keeps a pointer after the
  * call returns; all buffers, including fp32 gradient accumulators, belong to the
- * caller.  Return value: 0 on success, a negative LTR_E* code otherwise (nothing is
- * enqueued on error).  Re-entrant and safe to call from several host threads: the only
- * mutable global state is a small per-device record of facts found out on the first call
- * on each device (architecture check, large-LDS opt-in), kept in atomics and read-only
- * afterwards.
+ * caller (one exception, stated there: ltr_attn_bwd_noalloc keeps its DELTA workspace in
+ * a fixed array of its own).  Return value: 0 on success, a negative LTR_E* code otherwise
+ * (nothing is enqueued on error).  Re-entrant and safe to call from several host threads:
+ * the only mutable global state is a small per-device record of facts found out on the
+ * first call on each device (architecture check, large-LDS opt-in, address of the fixed
+ * scratch array), kept in atomics and read-only afterwards.
  *
  * Tensor layout: element strides (in elements, not bytes) are given for the batch,
  * sequence and head dimensions; the head dimension D is contiguous.  This serves
@@ -38,7 +39,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 3
+#define LTR_ABI_VERSION 4
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -61,6 +62,7 @@ extern "C" {
 #define LTR_EALIGN (-3)   /* pointer or stride not 16-byte aligned */
 #define LTR_ELAUNCH (-4)  /* HIP reported a launch error */
 #define LTR_EDEVICE (-5)  /* current device is not gfx950 */
+#define LTR_ETOOBIG (-6)  /* ltr_attn_bwd_noalloc: more rows than the fixed scratch holds */
 
 typedef struct ltr_kv_chunk {
     const void *k; /* [B, sk, Hkv, D] by kv strides */
@@ -177,6 +179,24 @@ typedef struct ltr_attn_bwd_args {
 } ltr_attn_bwd_args;
 
 int ltr_attn_bwd(const ltr_attn_bwd_args *args, void *stream);
+
+/*
+ * ltr_attn_bwd_noalloc - ltr_attn_bwd for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same arguments and results as ltr_attn_bwd with
+ * LTR_DELTA_FROM_O (which it implies: bf16 only, args->o required, LTR_NO_DQ refused), except
+ * that args->delta is IGNORED (may be NULL): the DELTA workspace is a fixed array of
+ * LTR_NOALLOC_MAX_ROWS floats (4 MiB) in device memory that belongs to the library; each
+ * GPU the library runs on holds its own copy until the process ends.  B * Hq * Sq must not
+ * exceed LTR_NOALLOC_MAX_ROWS (LTR_ETOOBIG otherwise).  The call allocates and frees
+ * nothing and calls no allocating routine.  All calls on one GPU share that GPU's array:
+ * two calls whose kernels may overlap on one GPU (different streams, different threads)
+ * race on it; calls on one stream are safe.  Every DELTA row a call's dK/dV kernel reads
+ * is written by its dQ kernel first, so nothing has to be cleared between calls.
+ */
+#define LTR_NOALLOC_MAX_ROWS (1 << 20)
+
+int ltr_attn_bwd_noalloc(const ltr_attn_bwd_args *args, void *stream);
 
 /* dst[i] = bf16(src[i]) (round to nearest even), i < n; both contiguous. */
 int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream);

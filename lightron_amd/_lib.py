@@ -7,12 +7,13 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
 
-LTR_ABI_VERSION = 3
+LTR_ABI_VERSION = 4
 LTR_MAX_CHUNKS = 32
+LTR_NOALLOC_MAX_ROWS = 1 << 20
 LTR_BF16, LTR_F32 = 0, 1
 LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LTR_DKDV_BF16 = 1, 2, 4, 8, 16, 32, 64
 
-EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
+EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_abi_version", "ltr_strerror")
 
 _i64x3 = ctypes.c_int64 * 3
@@ -84,6 +85,8 @@ def load():
     lib.ltr_attn_bwd_delta.restype = ctypes.c_int
     lib.ltr_attn_bwd.argtypes = [ctypes.POINTER(BwdArgs), ctypes.c_void_p]
     lib.ltr_attn_bwd.restype = ctypes.c_int
+    lib.ltr_attn_bwd_noalloc.argtypes = [ctypes.POINTER(BwdArgs), ctypes.c_void_p]
+    lib.ltr_attn_bwd_noalloc.restype = ctypes.c_int
     lib.ltr_cast_f32_to_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     lib.ltr_cast_f32_to_bf16.restype = ctypes.c_int
     lib.ltr_rope_apply.argtypes = [ctypes.POINTER(RopeArgs), ctypes.c_void_p]

@@ -130,7 +130,7 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
-                        causal=False, scale=None, do_dq=True, do_dkdv=True, o=None):
+                        causal=False, scale=None, do_dq=True, do_dkdv=True, o=None, library_scratch=False):
     """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
     do_dq / do_dkdv select which of the two backward kernels are enqueued.  dq_acc may instead be a bf16
     tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
@@ -138,8 +138,13 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     workspace: the dQ kernel of the first launch computes rowsum(dO * O) into it (LTR_DELTA_FROM_O) and no
     attn_delta call is needed; this needs do_dq.  dk_accs / dv_accs may be bf16 tensors as well: they then RECEIVE
     dK / dV (LTR_DKDV_BF16; every key is written), which is only right when q holds every query row that sees
-    these keys - one rank's own backward, not a ring step whose dK/dV are summed over ranks."""
+    these keys - one rank's own backward, not a ring step whose dK/dV are summed over ranks.
+    library_scratch=True calls ltr_attn_bwd_noalloc instead: delta is ignored (pass None), DELTA lives in the library's
+    fixed scratch array (at most LTR_NOALLOC_MAX_ROWS = B*Hq*Sq rows; calls that overlap on one GPU race on it), o is
+    required and the library allocates nothing."""
     lib = _lib.load()
+    if library_scratch and (o is None or not do_dq):
+        raise RuntimeError("library_scratch needs o (DELTA is computed from it) and do_dq")
     _req(q, "q")
     _req(do, "dO")
     B, Sq, Hq, D = q.shape
@@ -163,7 +168,8 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
         for t in list(dk_accs) + list(dv_accs):
             _req(t, "dK / dV")
     a = _lib.BwdArgs()
-    a.q, a.d_o, a.lse, a.delta, a.dq = q.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(), dq_acc.data_ptr()
+    a.q, a.d_o, a.lse, a.dq = q.data_ptr(), do.data_ptr(), lse.data_ptr(), dq_acc.data_ptr()
+    a.delta = None if library_scratch else delta.data_ptr()
     a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, ks[0].shape[2], D, Sq
     a.q_stride, a.do_stride, a.dq_stride = _s3(q), _s3(do), _s3(dq_acc)
     a.k_stride, a.v_stride = _s3(ks[0]), _s3(vs[0])
@@ -194,7 +200,10 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
                 ch.k, ch.v = ks[i].data_ptr(), vs[i].data_ptr()
                 ch.dk, ch.dv = dk_accs[i].data_ptr(), dv_accs[i].data_ptr()
                 ch.sk, ch.pos0 = ks[i].shape[1], int(k_pos0[i])
-            _lib.check(lib.ltr_attn_bwd(ctypes.byref(a), stream), "ltr_attn_bwd")
+            if library_scratch:
+                _lib.check(lib.ltr_attn_bwd_noalloc(ctypes.byref(a), stream), "ltr_attn_bwd_noalloc")
+            else:
+                _lib.check(lib.ltr_attn_bwd(ctypes.byref(a), stream), "ltr_attn_bwd")
 
 
 def cast_to_bf16(src: torch.Tensor) -> torch.Tensor:

@@ -1807,6 +1807,7 @@ constexpr int LTR_MAX_DEVICES = 64;
 struct DeviceState {
     std::atomic<int> arch{0};          // 0 unknown, 1 gfx950, -1 something else
     std::atomic<int> large_lds{0};     // 1: the kernels of this device may use more than 64 KB of dynamic LDS
+    std::atomic<float *> scratch{nullptr};   // device address of this device's copy of `scratch`
 };
 DeviceState g_dev[LTR_MAX_DEVICES];
 
@@ -1870,6 +1871,32 @@ bool strides_ok(const int64_t *s, int elem_bytes) {
 
 int fits_i32(int64_t x) { return x >= 0 && x < (int64_t)0x7fffffff; }
 
+// ------------------------------------------------------------------------------ fixed scratch
+// DELTA workspace of ltr_attn_bwd_noalloc: a fixed array in device memory that belongs to the library (every device the
+// library runs on holds its own copy until the process ends).  Host code never uses the array's name as an address: the
+// device address of the current device's copy is looked up once per device (scratch_address) and passed to the kernels
+// like any caller-owned workspace.
+}  // namespace
+static __device__ __align__(256) float scratch[LTR_NOALLOC_MAX_ROWS];
+namespace {
+
+int scratch_address(float **out) {
+    int dev = 0;
+    if (current_device(&dev)) return LTR_EDEVICE;
+    float *ptr = g_dev[dev].scratch.load(std::memory_order_acquire);
+    if (!ptr) {
+        void *sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) {
+            (void)hipGetLastError();
+            return LTR_ELAUNCH;
+        }
+        ptr = (float *)sym;
+        g_dev[dev].scratch.store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return LTR_OK;
+}
+
 }  // namespace
 
 extern "C" int ltr_abi_version(void) { return LTR_ABI_VERSION; }
@@ -1882,6 +1909,7 @@ extern "C" const char *ltr_strerror(int code) {
         case LTR_EALIGN: return "pointer or stride not 16-byte aligned";
         case LTR_ELAUNCH: return "HIP launch error";
         case LTR_EDEVICE: return "current device is not gfx950";
+        case LTR_ETOOBIG: return "size beyond the fixed scratch of the no-allocation entry point";
         default: return "unknown error";
     }
 }
@@ -1991,9 +2019,11 @@ extern "C" int ltr_attn_bwd_delta(const ltr_attn_delta_args *a, void *stream) {
 }
 
 namespace {
-int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, void *stream) {
-    float *delta = a->delta;
-    if (!a->q || !a->d_o || !a->lse || !delta) return LTR_EINVAL;
+// ltr_attn_bwd (DELTA is the caller's buffer) and ltr_attn_bwd_noalloc (use_scratch: DELTA lives in the library's fixed
+// scratch array; flags already carry LTR_DELTA_FROM_O)
+int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, void *stream) {
+    float *delta = use_scratch ? nullptr : a->delta;
+    if (!a->q || !a->d_o || !a->lse || (!use_scratch && !delta)) return LTR_EINVAL;
     const bool do_dq = !(flags & LTR_NO_DQ), do_dkdv = !(flags & LTR_NO_DKDV);
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
@@ -2039,6 +2069,10 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, void *stream) {
     }
     int rc = check_device();
     if (rc) return rc;
+    if (use_scratch) {
+        rc = scratch_address(&delta);
+        if (rc) return rc;
+    }
     p.q = a->q;
     p.d_o = a->d_o;
     p.lse = a->lse;
@@ -2109,7 +2143,18 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, void *stream) {
 
 extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (!a) return LTR_EINVAL;
-    return bwd_launch(a, a->flags, stream);
+    return bwd_launch(a, a->flags, false, stream);
+}
+
+extern "C" int ltr_attn_bwd_noalloc(const ltr_attn_bwd_args *a, void *stream) {
+    if (!a) return LTR_EINVAL;
+    if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;                 // DELTA comes from the bf16 forward output
+    if (a->flags & LTR_NO_DQ) return LTR_EINVAL;                    // the dQ kernel is the one that fills DELTA
+    if (a->B <= 0 || a->Hq <= 0 || a->Sq <= 0) return LTR_EINVAL;
+    if (a->Sq > LTR_NOALLOC_MAX_ROWS || (long long)a->B * a->Hq > LTR_NOALLOC_MAX_ROWS ||
+        (long long)a->B * a->Hq * a->Sq > LTR_NOALLOC_MAX_ROWS)
+        return LTR_ETOOBIG;
+    return bwd_launch(a, a->flags | LTR_DELTA_FROM_O, true, stream);
 }
 
 extern "C" int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void *stream) {

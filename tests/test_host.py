@@ -28,7 +28,7 @@ def test_header_symbols_exported():
     assert declared == set(L.EXPORTS), declared
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.ltr_abi_version() == 3
+    assert lib.ltr_abi_version() == 4
     assert lib.ltr_strerror(0) == b"ok" and b"aligned" in lib.ltr_strerror(-3)
 
 
@@ -77,6 +77,21 @@ def test_validation_without_gpu():
     assert lib.ltr_rope_apply(ctypes.byref(r), None) == -3          # 8-byte row stride in bf16
     r.x_stride[1], r.S = 32, 0
     assert lib.ltr_rope_apply(ctypes.byref(r), None) == 0           # empty input is a no-op
+
+
+def test_no_alloc_entry_point_validation_without_gpu():
+    L, lib = _lib()
+    assert lib.ltr_attn_bwd_noalloc(None, None) == -1
+    a = L.BwdArgs()
+    a.q = a.d_o = a.lse = a.dq = a.o = 4096
+    a.B, a.Hq, a.Hkv, a.D, a.n_chunks, a.io_dtype = 1, 32, 8, 128, 1, L.LTR_BF16
+    a.Sq = L.LTR_NOALLOC_MAX_ROWS // 32 + 1
+    assert lib.ltr_attn_bwd_noalloc(ctypes.byref(a), None) == -6      # more DELTA rows than the fixed scratch holds
+    assert b"scratch" in lib.ltr_strerror(-6)
+    a.Sq, a.flags = 64, L.LTR_NO_DQ
+    assert lib.ltr_attn_bwd_noalloc(ctypes.byref(a), None) == -1      # the dQ kernel is the one that fills DELTA
+    a.flags, a.io_dtype = 0, L.LTR_F32
+    assert lib.ltr_attn_bwd_noalloc(ctypes.byref(a), None) == -2      # bf16 only
 
 
 def test_missing_library_fails_loudly(monkeypatch):
