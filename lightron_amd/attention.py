@@ -222,7 +222,7 @@ class BlockAttentionFunction(torch.autograd.Function):
     fixed arguments are k_0..k_{n-1}, v_0..v_{n-1}."""
 
     @staticmethod
-    def forward(ctx, q, n_chunks, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, *kv):
+    def forward(ctx, q, n_chunks, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, kv_grad_acc, *kv):
         ks, vs = list(kv[:n_chunks]), list(kv[n_chunks:])
         if stepwise:
             # one launch per KV chunk, merged in the epilogue into an fp32 running (O, LSE)
@@ -236,6 +236,7 @@ class BlockAttentionFunction(torch.autograd.Function):
             o, lse = attn_fwd(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, out_dtype=out_dtype)
         ctx.save_for_backward(q, o, lse, *kv)
         ctx.meta = (n_chunks, list(k_pos0), q_pos0, q_split, causal, scale)
+        ctx.kv_grad_acc = kv_grad_acc
         ctx.mark_non_differentiable(lse)
         return o, lse
 
@@ -259,6 +260,14 @@ class BlockAttentionFunction(torch.autograd.Function):
         # one buffer per gradient, sliced along the sequence: every chunk's slice has the same strides.  This node's
         # q holds every query that sees these keys inside this node (autograd sums over nodes by itself), so for bf16
         # the kernels write dK / dV directly: no fp32 accumulators, no zero-fill, no cast.
+        if ctx.kv_grad_acc is not None:
+            # dK / dV of these chunks are summed over several nodes (the ranks of a ring) in caller-owned fp32
+            # accumulators and cast once at the end, instead of one bf16 rounding per node: nothing flows to k, v here
+            dk_accs, dv_accs = ctx.kv_grad_acc
+            attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal,
+                                scale, o=o if fuse else None)
+            dq = dq_acc if (direct or f32) else cast_to_bf16(dq_acc)
+            return (dq, None, None, None, None, None, None, None, None, None) + (None,) * (2 * n_chunks)
         lens = [k.shape[1] for k in ks]
         shape = (ks[0].shape[0], sum(lens), ks[0].shape[2], ks[0].shape[3])
         if f32:
@@ -276,12 +285,22 @@ class BlockAttentionFunction(torch.autograd.Function):
         dk16, dv16 = dk_buf, dv_buf
         dks = [dk16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         dvs = [dv16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
-        return (dq, None, None, None, None, None, None, None, None, *dks, *dvs)
+        return (dq, None, None, None, None, None, None, None, None, None, *dks, *dvs)
 
 
 def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, scale=None, stepwise=False,
-                    out_dtype=None):
-    """Differentiable entry: returns (O, LSE)."""
+                    out_dtype=None, kv_grad_acc=None):
+    """Differentiable entry: returns (O, LSE).  kv_grad_acc = (dk_accs, dv_accs), fp32 tensors shaped like ks / vs:
+    the backward then ADDS dK / dV into them (no gradient flows to ks / vs through autograd); the owner of the
+    accumulators makes the one final cast.  That is how a ring sums dK / dV over its ranks without a bf16 rounding
+    per rank."""
     n = len(ks)
+    if kv_grad_acc is not None:
+        dk_accs, dv_accs = kv_grad_acc
+        if len(dk_accs) != n or len(dv_accs) != n:
+            raise RuntimeError("kv_grad_acc needs one dK and one dV accumulator per KV chunk")
+        for a, k in zip(list(dk_accs) + list(dv_accs), list(ks) + list(vs)):
+            if a.dtype != torch.float32 or a.shape != k.shape:
+                raise RuntimeError("kv_grad_acc entries must be fp32 tensors shaped like their chunks")
     return BlockAttentionFunction.apply(q, n, list(k_pos0), q_pos0, q_split, causal, scale, stepwise, out_dtype,
-                                        *ks, *vs)
+                                        kv_grad_acc, *ks, *vs)

@@ -17,6 +17,36 @@ import torch
 from .attention import block_attention
 
 
+class RingKVGrads:
+    """fp32 dK / dV accumulators of a ring whose KV chunks live on this GPU, shared by the LocalRing descriptors of all
+    its ranks: every rank's backward adds its contribution (the kernels accumulate in fp32), and finalize() makes the
+    ONE cast to the chunks' dtype.  Without it autograd sums W bf16-rounded per-rank gradients.  In a real ring these
+    are the accumulators that travel with the KV chunk."""
+
+    def __init__(self, kv: Sequence):
+        self.kv = list(kv)
+        self.dk = [torch.zeros(k.shape, dtype=torch.float32, device=k.device) for k, _ in self.kv]
+        self.dv = [torch.zeros(v.shape, dtype=torch.float32, device=v.device) for _, v in self.kv]
+
+    def zero_(self):
+        for t in self.dk + self.dv:
+            t.zero_()
+
+    def finalize(self, assign: bool = True):
+        """[(dK, dV)] per rank in the chunks' dtype; with assign=True also added to k.grad / v.grad of leaf tensors."""
+        from .attention import cast_to_bf16
+        out = []
+        for (k, v), dk, dv in zip(self.kv, self.dk, self.dv):
+            gk = cast_to_bf16(dk) if k.dtype == torch.bfloat16 else dk.to(k.dtype)
+            gv = cast_to_bf16(dv) if v.dtype == torch.bfloat16 else dv.to(v.dtype)
+            if assign:
+                for t, g in ((k, gk), (v, gv)):
+                    if t.requires_grad and t.is_leaf:
+                        t.grad = g.clone() if t.grad is None else t.grad + g
+            out.append((gk, gv))
+        return out
+
+
 class LocalRing:
     """Stand-in for the cp ProcessGroup of a ring whose KV chunks all live on this GPU.
 
@@ -31,10 +61,13 @@ class LocalRing:
                        epilogue (the shape of a real ring, where chunks arrive one at a
                        time) instead of one launch that walks the whole chunk table.
     out_dtype        : dtype of the result (default: dtype of local_q).
+    kv_grads         : a RingKVGrads over the same kv list, shared by all ranks' descriptors: the backward adds dK / dV
+                       into its fp32 accumulators instead of returning per-rank gradients to autograd.
     """
 
     def __init__(self, rank: int, world_size: int, kv: Optional[Sequence] = None, causal: bool = False,
-                 layout: str = "contiguous", stepwise: bool = False, out_dtype: Optional[torch.dtype] = None):
+                 layout: str = "contiguous", stepwise: bool = False, out_dtype: Optional[torch.dtype] = None,
+                 kv_grads: Optional[RingKVGrads] = None):
         if not (0 <= rank < world_size):
             raise ValueError("rank %d outside ring of %d" % (rank, world_size))
         if layout not in ("contiguous", "zigzag"):
@@ -44,6 +77,9 @@ class LocalRing:
         if len(self.kv) != world_size:
             raise ValueError("kv must have one entry per rank")
         self.causal, self.layout, self.stepwise, self.out_dtype = causal, layout, stepwise, out_dtype
+        if kv_grads is not None and len(kv_grads.dk) != world_size:
+            raise ValueError("kv_grads must cover one KV chunk per rank")
+        self.kv_grads = kv_grads
         self.last_lse = None
 
     def order(self) -> List[int]:
@@ -55,6 +91,8 @@ def _chunk_table(ring: LocalRing, local_k, local_v, s_local: int):
     """KV chunks in visiting order with the global position of each chunk's first key."""
     W = ring.world_size
     ks, vs, pos = [], [], []
+    dks, dvs = [], []
+    acc = ring.kv_grads
     for j in ring.order():
         kv = ring.kv[j]
         if kv is None:
@@ -66,12 +104,18 @@ def _chunk_table(ring: LocalRing, local_k, local_v, s_local: int):
             ks.append(k)
             vs.append(v)
             pos.append(j * s_local)
+            if acc is not None:
+                dks.append(acc.dk[j])
+                dvs.append(acc.dv[j])
         else:
             hc = s_local // 2
             ks += [k[:, :hc], k[:, hc:]]
             vs += [v[:, :hc], v[:, hc:]]
             pos += [j * hc, (2 * W - 1 - j) * hc]
-    return ks, vs, pos
+            if acc is not None:
+                dks += [acc.dk[j][:, :hc], acc.dk[j][:, hc:]]
+                dvs += [acc.dv[j][:, :hc], acc.dv[j][:, hc:]]
+    return ks, vs, pos, ((dks, dvs) if acc is not None else None)
 
 
 def ring_attention_with_lse(local_q, local_k, local_v, cp_group) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -97,9 +141,11 @@ def ring_attention_with_lse(local_q, local_k, local_v, cp_group) -> Tuple[torch.
         q_pos0, q_split = (ring.rank * hc, (2 * W - 1 - ring.rank) * hc), hc
     else:
         q_pos0, q_split = (ring.rank * S_local, ring.rank * S_local), S_local
-    ks, vs, pos = _chunk_table(ring, local_k, local_v, S_local)
+    ks, vs, pos, grad_acc = _chunk_table(ring, local_k, local_v, S_local)
+    if grad_acc is not None and ring.kv[ring.rank] is None:
+        raise RuntimeError("kv_grads needs the ring's own chunk in LocalRing.kv (entry %d is None)" % ring.rank)
     o, lse = block_attention(local_q, ks, vs, pos, q_pos0, q_split, ring.causal, None, ring.stepwise,
-                             ring.out_dtype)
+                             ring.out_dtype, grad_acc)
     return o, lse
 
 

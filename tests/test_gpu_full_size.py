@@ -71,9 +71,13 @@ def test_config2_full(ltr):
     assert (outs[0][1] - outs[1][1]).abs().max() < 1e-3     # l sums bf16-rounded P: order-dependent rounding
 
 
-def test_config3_full_all_ranks(ltr):
+@pytest.mark.parametrize("path", ["accumulators", "bench"])
+def test_config3_full_all_ranks(ltr, path):
     """B=1, Hq=32, Hkv=8, D=128, S=32768 as 8 zig-zag rank shares, bf16, causal, N(0,1) seed 0:
-    O, LSE, dQ, dK, dV of the whole sequence."""
+    O, LSE, dQ, dK, dV of the whole sequence.  path "accumulators": separate DELTA launch, fp32 dQ accumulator, one
+    backward call; path "bench": exactly the call sequence bench.py times - a dQ-only call that computes DELTA from O
+    into a shared workspace and writes bf16 dQ (LTR_DELTA_FROM_O | LTR_DQ_BF16), then a dK/dV-only call that reads
+    that workspace."""
     g = torch.Generator().manual_seed(0)
     B, Hq, Hkv, D, S, W = 1, 32, 8, 128, 32768, 8
     mk = lambda h: torch.randn(B, S, h, D, generator=g).to(torch.bfloat16)
@@ -88,6 +92,7 @@ def test_config3_full_all_ranks(ltr):
     o = torch.empty_like(qd)
     lse = torch.empty(B, Hq, S, device="cuda")
     dq = torch.empty(qd.shape, dtype=torch.float32, device="cuda")
+    delta_ws = torch.empty(B, Hq, sl, dtype=torch.float32, device="cuda")       # one workspace for all shares, as in bench.py
     for r in range(W):
         idx = rp[r].cuda()
         ql, dol = qd[:, idx].contiguous(), dod[:, idx].contiguous()
@@ -100,10 +105,15 @@ def test_config3_full_all_ranks(ltr):
             pos += [j * hc, (2 * W - 1 - j) * hc]
         qp = (r * hc, (2 * W - 1 - r) * hc)
         ol, lsel = ltr.attn_fwd(ql, ks, vs, pos, qp, hc, True)
-        delta = ltr.attn_delta(ol, dol)
-        dql = torch.zeros(ql.shape, dtype=torch.float32, device="cuda")
-        ltr.attn_bwd_accumulate(ql, dol, lsel, delta, ks, vs, pos, dql, dks, dvs, qp, hc, True)
-        o[:, idx], dq[:, idx], lse[:, :, idx] = ol, dql, lsel
+        if path == "bench":
+            dql = torch.empty(ql.shape, dtype=torch.bfloat16, device="cuda")
+            ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos, dql, dks, dvs, qp, hc, True, do_dkdv=False, o=ol)
+            ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos, dql, dks, dvs, qp, hc, True, do_dq=False)
+        else:
+            delta = ltr.attn_delta(ol, dol)
+            dql = torch.zeros(ql.shape, dtype=torch.float32, device="cuda")
+            ltr.attn_bwd_accumulate(ql, dol, lsel, delta, ks, vs, pos, dql, dks, dvs, qp, hc, True)
+        o[:, idx], dq[:, idx], lse[:, :, idx] = ol, dql.float(), lsel
     dk = torch.empty(kd.shape, dtype=torch.float32, device="cuda")
     dv = torch.empty(vd.shape, dtype=torch.float32, device="cuda")
     for r in range(W):
@@ -118,10 +128,44 @@ def test_config3_full_all_ranks(ltr):
     assert _rel(lhs, rhs) < 1e-2
 
 
-def test_config4_full_rank15(ltr):
+def test_config3_full_ring_entry_point_fp32_kv_grads(ltr):
+    """The same workload through the drop-in entry point: ring_attention_kernel with a LocalRing per rank (W = 8,
+    zig-zag) and autograd, dK / dV summed over the 8 ranks in the ring's fp32 accumulators (RingKVGrads) and cast
+    once."""
+    g = torch.Generator().manual_seed(0)
+    B, Hq, Hkv, D, S, W = 1, 32, 8, 128, 32768, 8
+    mk = lambda h: torch.randn(B, S, h, D, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    rp = [orc.zigzag_positions(r, W, S) for r in range(W)]
+    kv = [(k[:, p].cuda().requires_grad_(True), v[:, p].cuda().requires_grad_(True)) for p in rp]
+    grads = ltr.RingKVGrads(kv)
+    o = torch.empty(B, S, Hq, D, dtype=torch.bfloat16)
+    lse = torch.empty(B, Hq, S)
+    dq = torch.empty(B, S, Hq, D, dtype=torch.bfloat16)
+    for r in range(W):
+        ql = q[:, rp[r]].cuda().requires_grad_(True)
+        ring = ltr.LocalRing(r, W, kv, causal=True, layout="zigzag", kv_grads=grads)
+        ol = ltr.ring_attention_kernel(ql, kv[r][0], kv[r][1], ring, None)
+        ol.backward(do[:, rp[r]].cuda())
+        o[:, rp[r]], lse[:, :, rp[r]], dq[:, rp[r]] = ol.detach().cpu(), ring.last_lse.cpu(), ql.grad.cpu()
+        assert kv[r][0].grad is None                      # nothing reaches k / v before finalize()
+    grads.finalize()
+    dk = torch.empty(B, S, Hkv, D, dtype=torch.bfloat16)
+    dv = torch.empty(B, S, Hkv, D, dtype=torch.bfloat16)
+    for r in range(W):
+        dk[:, rp[r]], dv[:, rp[r]] = kv[r][0].grad.cpu(), kv[r][1].grad.cpu()
+    pos = torch.arange(S)
+    _check_rows(q, k, v, pos, pos, True, o, lse, do, dq, n=20, seed=3)
+    _check_keys(q, k, v, o, lse, do, pos, pos, True, dk, dv, n=6, seed=4)
+    rhs = do.double().sum(1).reshape(B, Hkv, Hq // Hkv, D).sum(2)
+    assert _rel(dv.double().sum(1), rhs) < 1e-2
+
+
+@pytest.mark.parametrize("path", ["accumulators", "bench"])
+def test_config4_full_rank15(ltr, path):
     """B=1, H=8, D=128, S=131072 as 16 chunks of 8192, bf16, causal, RoPE (base 10000) applied to
     q and k beforehand; rank 15's Q chunk against all 16 KV chunks: O, LSE, dQ and this rank's
-    contribution to dK, dV of every chunk."""
+    contribution to dK, dV of every chunk.  The two paths are those of test_config3_full_all_ranks."""
     g = torch.Generator().manual_seed(0)
     B, H, D, S, W = 1, 8, 128, 131072, 16
     sl = S // W
@@ -150,13 +194,19 @@ def test_config4_full_rank15(ltr):
     vs = [vd[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
     pos0 = [j * sl for j in orc.ring_order(15, W)]
     ol, lsel = ltr.attn_fwd(ql, ks, vs, pos0, 15 * sl, None, True)
-    delta = ltr.attn_delta(ol, dol)
-    dq = torch.zeros(ql.shape, dtype=torch.float32, device="cuda")
     dk = torch.zeros(kd.shape, dtype=torch.float32, device="cuda")
     dv = torch.zeros(vd.shape, dtype=torch.float32, device="cuda")
     dks = [dk[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
     dvs = [dv[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
-    ltr.attn_bwd_accumulate(ql, dol, lsel, delta, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True)
+    if path == "bench":
+        dq = torch.empty(ql.shape, dtype=torch.bfloat16, device="cuda")
+        delta_ws = torch.empty(B, H, sl, dtype=torch.float32, device="cuda")
+        ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True, do_dkdv=False, o=ol)
+        ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True, do_dq=False)
+    else:
+        delta = ltr.attn_delta(ol, dol)
+        dq = torch.zeros(ql.shape, dtype=torch.float32, device="cuda")
+        ltr.attn_bwd_accumulate(ql, dol, lsel, delta, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True)
     qpos, kpos = torch.arange(sl) + 15 * sl, torch.arange(S)
     qc = q[:, 15 * sl:]
     oc, lsec = ol.cpu(), lsel.cpu()

@@ -672,6 +672,87 @@ def test_ring_sweep_all_ranks_forward_backward(ltr, seed):
     assert _rel(dk, dk_ref) < GRAD_RTOL_BF16 and _rel(dv, dv_ref) < GRAD_RTOL_BF16
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_ring_fp32_kv_grads_one_cast(ltr, seed):
+    """RingKVGrads: dK / dV summed over the ranks in fp32 and cast once.  Against the dense gradients, and closer to them
+    (or as close) than the sum of per-rank bf16 gradients; nothing reaches k.grad before finalize()."""
+    import random
+    rnd = random.Random(7100 + seed)
+    g = torch.Generator().manual_seed(8100 + seed)
+    W, layout = rnd.choice([2, 4, 6]), rnd.choice(["contiguous", "zigzag"])
+    D, Hkv, Hq, B, Sl = rnd.choice([64, 128]), 2, 4, rnd.choice([1, 2]), rnd.choice([64, 130, 256])
+    S = W * Sl
+    q, do = (_randn((B, S, Hq, D), g, torch.bfloat16) for _ in range(2))
+    k, v = (_randn((B, S, Hkv, D), g, torch.bfloat16) for _ in range(2))
+    pos = torch.arange(S)
+    _, _, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), k.float(), v.float(), do.float(), pos, pos, True)
+    share = [orc.zigzag_positions(r, W, S) if layout == "zigzag" else orc.contiguous_positions(r, Sl) for r in range(W)]
+    errs = {}
+    for mode in ("fp32", "bf16"):
+        kd = [k[:, share[r]].contiguous().cuda().requires_grad_(True) for r in range(W)]
+        vd = [v[:, share[r]].contiguous().cuda().requires_grad_(True) for r in range(W)]
+        kv = list(zip(kd, vd))
+        grads = ltr.RingKVGrads(kv) if mode == "fp32" else None
+        for r in range(W):
+            qr = q[:, share[r]].contiguous().cuda().requires_grad_(True)
+            ring = ltr.LocalRing(r, W, kv=kv, causal=True, layout=layout, kv_grads=grads)
+            ltr.ring_attention_kernel(qr, kd[r], vd[r], ring, None).backward(do[:, share[r]].contiguous().cuda())
+            assert _rel(qr.grad.cpu(), dq_ref[:, share[r]]) < GRAD_RTOL_BF16
+        if grads is not None:
+            assert all(t.grad is None for t in kd + vd)
+            grads.finalize()
+        dk, dv = torch.zeros_like(dk_ref), torch.zeros_like(dv_ref)
+        for r in range(W):
+            dk[:, share[r]], dv[:, share[r]] = kd[r].grad.cpu().double(), vd[r].grad.cpu().double()
+        errs[mode] = (_rel(dk, dk_ref), _rel(dv, dv_ref))
+        assert max(errs[mode]) < GRAD_RTOL_BF16
+    assert errs["fp32"][0] <= errs["bf16"][0] * 1.05 and errs["fp32"][1] <= errs["bf16"][1] * 1.05, errs
+
+
+@pytest.mark.parametrize("dtype,n_chunks", [(torch.bfloat16, 40), (torch.bfloat16, 70), (torch.float32, 35)])
+def test_more_chunks_than_one_launch_holds(ltr, dtype, n_chunks):
+    """More KV chunks than one launch's table (32): the host splits them into several launches.  Forward: the later
+    launches merge into the (O, LSE) of the earlier ones (LTR_MERGE); backward: DELTA from O on the first launch only, dQ
+    accumulated in fp32 over the launches and cast, dK / dV of each launch's chunks written by it.  Ragged chunk lengths
+    of 16-64 keys, GQA, causal with the chunks' positions shuffled, through block_attention and autograd, against the
+    dense oracle."""
+    import random
+    rnd = random.Random(4200 + n_chunks)
+    g = torch.Generator().manual_seed(4300 + n_chunks)
+    B, Hq, Hkv, D = 2, 4, 2, 128 if dtype == torch.bfloat16 else 64
+    lens = [rnd.randint(16, 64) for _ in range(n_chunks)]
+    starts = [sum(lens[:i]) for i in range(n_chunks)]
+    Sk = sum(lens)
+    Sq = 200
+    q_pos0 = Sk - Sq - 37                                # the last keys are invisible to every query
+    q, do = (_randn((B, Sq, Hq, D), g, dtype) for _ in range(2))
+    k, v = (_randn((B, Sk, Hkv, D), g, dtype) for _ in range(2))
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(
+        q.float(), k.float(), v.float(), do.float(), torch.arange(Sq) + q_pos0, torch.arange(Sk), True)
+    order = list(range(n_chunks))
+    rnd.shuffle(order)                                   # visiting order != position order
+    qd = q.cuda().requires_grad_(True)
+    kl = [k[:, starts[j]:starts[j] + lens[j]].contiguous().cuda().requires_grad_(True) for j in order]
+    vl = [v[:, starts[j]:starts[j] + lens[j]].contiguous().cuda().requires_grad_(True) for j in order]
+    o, lse = ltr.block_attention(qd, kl, vl, [starts[j] for j in order], q_pos0, None, True)
+    o.backward(do.cuda())
+    f32 = dtype == torch.float32
+    assert (o.detach().cpu().double() - o_ref).abs().max() < (F32_TOL if f32 else O_TOL_BF16)
+    assert (lse.cpu().double() - lse_ref).abs().max() < (F32_TOL if f32 else LSE_TOL_BF16)
+    dk, dv = torch.zeros_like(dk_ref), torch.zeros_like(dv_ref)
+    for i, j in enumerate(order):
+        dk[:, starts[j]:starts[j] + lens[j]] = kl[i].grad.cpu().double()
+        dv[:, starts[j]:starts[j] + lens[j]] = vl[i].grad.cpu().double()
+    if f32:
+        assert (qd.grad.cpu().double() - dq_ref).abs().max() < F32_TOL * max(1.0, dq_ref.abs().max().item())
+        assert (dk - dk_ref).abs().max() < F32_TOL * max(1.0, dk_ref.abs().max().item())
+        assert (dv - dv_ref).abs().max() < F32_TOL * max(1.0, dv_ref.abs().max().item())
+    else:
+        assert _rel(qd.grad.cpu(), dq_ref) < GRAD_RTOL_BF16
+        assert _rel(dk, dk_ref) < GRAD_RTOL_BF16 and _rel(dv, dv_ref) < GRAD_RTOL_BF16
+    assert dk[:, q_pos0 + Sq:].abs().max() == 0 and dv[:, q_pos0 + Sq:].abs().max() == 0    # keys no query sees
+
+
 @pytest.mark.parametrize("seed", list(range(8)))
 def test_rope_sweep_bit_exact(ltr, seed):
     """ltr_rope_apply on random shapes, dtypes, layouts and starting positions against the oracle, bit for bit."""

@@ -147,7 +147,7 @@ def test_ring_descriptor_order_and_positions():
     from lightron_amd.ring_attention import LocalRing, _chunk_table
     ring = LocalRing(2, 4, kv=[(torch.zeros(1, 8, 1, 4), torch.zeros(1, 8, 1, 4))] * 4, layout="zigzag")
     assert ring.order() == orc.ring_order(2, 4) == [2, 1, 0, 3]
-    ks, vs, pos = _chunk_table(ring, None, None, 8)
+    ks, vs, pos, _ = _chunk_table(ring, None, None, 8)
     exp = []
     for j in ring.order():
         p = orc.zigzag_positions(j, 4, 32)
