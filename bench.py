@@ -21,9 +21,28 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 matrix peak
-# HBM-side bytes per launch of bwd_dkdv_kernel<128> on config 3, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
-# command calibrated against streaming kernels of known size (profiles/bench_c3_counters.md)
-DKDV_C3_TRAFFIC_BYTES = 2.30e9
+KERNEL_SOURCE = os.path.join(ROOT, "lightron_amd", "csrc", "ltr_attn.hip")
+COUNTER_PROFILE = os.path.join(ROOT, "profiles", "bench_c3_counters.md")
+
+
+def _measured_traffic(kernel):
+    """HBM-side bytes per launch of `kernel` on config 3 as the rocprofv3 FETCH_SIZE / WRITE_SIZE runs recorded in
+    profiles/bench_c3_counters.md measured them.  The profile names the sha256 of the kernel source it was taken from;
+    when the source has changed since, the figure is stale and None is reported instead."""
+    import hashlib
+    import re
+    try:
+        text = open(COUNTER_PROFILE).read()
+        digest = hashlib.sha256(open(KERNEL_SOURCE, "rb").read()).hexdigest()
+    except OSError:
+        return None, "no counter profile"
+    m = re.search(r"^kernel-source-sha256: ([0-9a-f]{64})$", text, flags=re.M)
+    t = re.search(r"^traffic-bytes-per-launch %s: ([0-9.e+]+)$" % re.escape(kernel), text, flags=re.M)
+    if not m or not t:
+        return None, "profiles/bench_c3_counters.md has no machine-readable traffic line for %s" % kernel
+    if m.group(1) != digest:
+        return None, "profiles/bench_c3_counters.md was taken from an older kernel source (stale)"
+    return float(t.group(1)), "profiles/bench_c3_counters.md (rocprofv3 FETCH_SIZE/WRITE_SIZE, source sha256 %s)" % digest[:12]
 
 
 def _workload(name):
@@ -44,6 +63,10 @@ def _workload(name):
         return dict(B=8, Hq=4, Hkv=4, D=64, S=4096, W=1, layout="contiguous", causal=False,
                     ranks=[0], bwd=True,
                     desc="config 5: B=8, 4 local heads of 16, D=64, S=4096, non-causal, fwd+bwd")
+    if name == "s2k":
+        return dict(B=8, Hq=32, Hkv=32, D=128, S=2048, W=1, layout="contiguous", causal=True,
+                    ranks=[0], bwd=True,
+                    desc="single-chunk causal attention (the Attention.forward / Ulysses local shape): B=8 H=32 D=128 S=2048, fwd+bwd")
     raise SystemExit("unknown workload %r" % name)
 
 
@@ -146,26 +169,53 @@ def _bench_rope(args):
     print(json.dumps(out), flush=True)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "rope"])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        raise SystemExit("bench.py: this build runs on ONE GPU (no collectives, no sharding across GPUs); "
-                         "run with --gpus 1")
-    import torch
-    import lightron_amd as la
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    if args.workload == "rope":
-        return _bench_rope(args)
-    la._lib.load()
-    torch.cuda.set_device(0)
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _device_report(la, torch, probe=True):
+    """hipDeviceProp facts of the device plus what it sustains on the matrix pipe right now: a register-resident
+    v_mfma_f32_32x32x16_bf16 loop on random and on constant operands, with the shader clock measured inside each."""
+    import ctypes
+    lib = la._lib.load()
+    info = la._lib.DeviceInfo()
+    la._lib.check(lib.ltr_device_info(ctypes.byref(info)), "ltr_device_info")
+    rep = {"name": torch.cuda.get_device_properties(0).name, "arch": info.arch.decode(), "cus": info.compute_units,
+           "clock_mhz": info.clock_khz // 1000, "memory_clock_mhz": info.memory_clock_khz // 1000,
+           "memory_bus_bits": info.memory_bus_bits, "hbm_gib": round(info.hbm_bytes / 2**30, 1)}
+    if not probe:
+        return rep
+    n = 8192 + (1 << 20)
+    g = torch.Generator().manual_seed(1)
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    ws[8192:] = ((torch.rand((n - 8192) // 2, generator=g) * 4 - 2).to(torch.bfloat16)).view(torch.uint8).cuda()
+    iters = 200000
+    stream = torch.cuda.current_stream().cuda_stream
+    for key, rnd in (("random_operands", 1), ("constant_operands", 0)):
+        best = None
+        for _ in range(2):      # the first launch also ramps the clock
+            la._lib.check(lib.ltr_probe_mfma(ws.data_ptr(), n, iters, rnd, stream), "ltr_probe_mfma")
+            torch.cuda.synchronize()
+            t = ws[:16].view(torch.int64).cpu()
+            sec = t[0].item() / 100e6
+            cur = {"tflops": round(info.compute_units * 8 * iters * 4 * 32768.0 / sec / 1e12, 1),
+                   "shader_clock_mhz": round(t[1].item() / sec / 1e6, 0)}
+            best = cur if best is None or cur["tflops"] > best["tflops"] else best
+        rep["mfma_loop_" + key] = best
+    return rep
+
+
+def _run_attention(la, torch, cfg, steps, warmup):
+    """Times `steps` steps of one workload after `warmup` untimed ones; inputs are resident in HBM before the timed
+    region.  Returns the step time, the credited flops and the average launch time of each kernel (HIP events on the
+    stream the kernels are launched on)."""
     dev = torch.device("cuda:0")
-    cfg = _workload(args.workload)
     B, Hq, Hkv, D, S, W = (cfg[x] for x in ("B", "Hq", "Hkv", "D", "S", "W"))
     causal, bwd = cfg["causal"], cfg["bwd"]
     sl = S // W
@@ -181,7 +231,7 @@ def main():
     # per-rank chunk tables in the reference's visiting order
     tables = {}
     for r in cfg["ranks"]:
-        ks, vs, dks, dvs, pos = [], [], [], [], []
+        ks, vs, pos = [], [], []
         for j in [(r - s) % W for s in range(W)]:
             if cfg["layout"] == "zigzag":
                 hc = sl // 2
@@ -250,19 +300,18 @@ def main():
         if bwd and not dkdv_direct:
             la.cast_to_bf16(dk_acc); la.cast_to_bf16(dv_acc)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step(False)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step(True)
     torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    dt = (time.perf_counter() - t0) / steps
 
     pairs = sum(_n_pairs(cfg, r) for r in cfg["ranks"])
     f_fwd = 4.0 * B * Hq * D * pairs
     f_total = f_fwd * (3.5 if bwd else 1.0)
-    tflops = f_total / dt / 1e12
     avg = lambda key: sum(a.elapsed_time(b) for a, b in ev[key]) / len(ev[key])
     fwd_ms = avg("fwd")
     launches = len(cfg["ranks"])
@@ -280,27 +329,108 @@ def main():
         dom, dom_ms, dom_flops = "bwd_dkdv_kernel<%d>" % D, dkdv_ms, 2.0 * f_share
     else:
         dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_share
-    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
-    prop = torch.cuda.get_device_properties(0)
+    return {"dt": dt, "f_total": f_total, "kernels": kernels, "launches": launches,
+            "dominant": (dom, dom_flops / (dom_ms * 1e-3) / 1e12)}
+
+
+def _bench_mfma_ceiling(args):
+    """What the device sustains on the matrix pipe, for the record beside the attention numbers: the register-resident
+    MFMA loop of ltr_probe_mfma on random and constant operands with the shader clock of each, and the vendor library's
+    bf16 GEMM (torch.matmul, 8192^3) on N(0,1) inputs."""
+    import torch
+    import lightron_amd as la
+    torch.cuda.set_device(0)
+    rep = _device_report(la, torch)
+    a = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    for _ in range(5):
+        a @ b
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        a @ b
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    rep["library_gemm_bf16_8192"] = {"tflops": round(2 * 8192.0**3 / ms / 1e9, 1), "ms": round(ms, 4)}
+    best = rep["mfma_loop_random_operands"]["tflops"]
+    out = {"metric": "sustained bf16 MFMA rate of the device (register-resident v_mfma_f32_32x32x16_bf16 loop, random operands)",
+           "value": best, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "matrix-pipe ceiling probe: one block of 8 waves per CU, 4 MFMA chains per wave"},
+           "frac_of_mfma_peak": round(best / MFMA_BF16_PEAK_TFLOPS, 4), "device": rep}
+    print(json.dumps(out), flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other workloads and the device probe")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (no collectives, no sharding across GPUs); "
+                         "run with --gpus 1")
+    import torch
+    import lightron_amd as la
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.workload == "rope":
+        return _bench_rope(args)
+    if args.workload == "mfma_ceiling":
+        return _bench_mfma_ceiling(args)
+    la._lib.load()
+    torch.cuda.set_device(0)
+    cfg = _workload(args.workload)
+    res = _run_attention(la, torch, cfg, args.steps, args.warmup)
+    dt, f_total, bwd = res["dt"], res["f_total"], cfg["bwd"]
+    tflops = f_total / dt / 1e12
+    dom, achieved = res["dominant"]
+    traffic, traffic_source = (None, None)
+    if args.workload == "c3":
+        traffic, traffic_source = _measured_traffic(dom)
     out = {
         "metric": ("ring-attn fwd+bwd causal TFLOP/s at S=32k bf16, 1 GPU; % of MFMA peak" if args.workload == "c3" else
                    "attention %s causal-adjusted TFLOP/s, 1 GPU; %% of MFMA peak" % ("fwd+bwd" if bwd else "fwd")),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": cfg["desc"], "B": B, "Hq": Hq, "Hkv": Hkv, "D": D, "S": S, "ranks": launches,
-                   "layout": cfg["layout"], "causal": causal, "flops_per_step": f_total},
+        "config": {"workload": cfg["desc"], "B": cfg["B"], "Hq": cfg["Hq"], "Hkv": cfg["Hkv"], "D": cfg["D"], "S": cfg["S"],
+                   "ranks": res["launches"], "layout": cfg["layout"], "causal": cfg["causal"], "flops_per_step": f_total},
         "frac_of_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        "kernels": kernels,
+        "kernels": res["kernels"],
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": DKDV_C3_TRAFFIC_BYTES if (args.workload == "c3" and bwd) else None},
-        "device": {"name": prop.name, "cus": prop.multi_processor_count,
-                   "clock_mhz": getattr(prop, "clock_rate", 0) // 1000},
+                     "traffic": traffic, "traffic_source": traffic_source},
     }
+    if not args.no_others:
+        # the other workloads, outside the timed region of the headline: a few steps each
+        others = {}
+        for name in ("c2", "c4", "c5", "s2k"):
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            ocfg = _workload(name)
+            r = _run_attention(la, torch, ocfg, 5, 2)
+            tf = r["f_total"] / r["dt"] / 1e12
+            others[name] = {"workload": ocfg["desc"], "tflops": round(tf, 1), "ms_per_step": round(r["dt"] * 1e3, 3),
+                            "frac_of_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                            "kernel_ms": {k: v["ms_per_launch"] for k, v in r["kernels"].items()},
+                            "dominant_kernel_frac": round(r["dominant"][1] / MFMA_BF16_PEAK_TFLOPS, 4)}
+        out["other_workloads"] = others
+    out["device"] = _device_report(la, torch, probe=not args.no_others)
     if not args.no_cpu_baseline:
-        threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-        out["cpu_baseline"] = _cpu_baseline(cfg, threads)
+        # the host's cores as the box presents them; OMP_NUM_THREADS (set on the GPU boxes to the job's CPU share) caps
+        # the threads actually used
+        host_cores = os.cpu_count() or 1
+        threads = int(os.environ["OMP_NUM_THREADS"]) if os.environ.get("OMP_NUM_THREADS", "").isdigit() else host_cores
+        threads = max(1, min(threads, host_cores))
+        base = _cpu_baseline(cfg, threads)
+        base.update({"threads": threads, "host_cores": host_cores, "cpu_model": _cpu_model()})
+        out["cpu_baseline"] = base
     print(json.dumps(out), flush=True)
 
 

@@ -229,6 +229,35 @@ typedef struct ltr_rope_args {
 
 int ltr_rope_apply(const ltr_rope_args *args, void *stream);
 
+/*
+ * Measurement helpers (no counterpart in the reference: its only performance output is a printed wall time,
+ * ring_attention.py:195-196).  A benchmark prints the kernels' rates beside what the device itself sustains.
+ *
+ * ltr_device_info - facts of the CURRENT device as hipDeviceProp reports them (host call, nothing is enqueued).
+ *
+ * ltr_probe_mfma - enqueues one kernel in which every wave of every CU (one block of 8 waves per CU) runs
+ * 4 * iters v_mfma_f32_32x32x16_bf16 on register-resident operands: the device's matrix-pipe ceiling.
+ * random_operands != 0: the operands are read once from workspace bytes [8192, workspace_bytes), which the caller
+ * fills (random bf16 data makes the chip run at the clock its power limit allows); 0: constant operands.
+ * Results, valid once the stream has finished: ((int64_t *)workspace)[0] = elapsed ticks of the constant 100 MHz
+ * wall clock, [1] = elapsed ticks of the shader clock counter.  Rate = CUs * 8 * iters * 4 * 32768 flop / seconds.
+ * workspace: device memory, 16-byte aligned, at least LTR_PROBE_MIN_WORKSPACE bytes.
+ */
+typedef struct ltr_device_info_t {
+    int32_t compute_units;
+    int32_t clock_khz;            /* hipDeviceProp.clockRate: the engine clock the device advertises */
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    int64_t lds_bytes_per_block;
+    int64_t hbm_bytes;
+    char arch[64];
+} ltr_device_info_t;
+
+#define LTR_PROBE_MIN_WORKSPACE (8192 + 65536)
+
+int ltr_device_info(ltr_device_info_t *out);
+int ltr_probe_mfma(void *workspace, int64_t workspace_bytes, int32_t iters, int32_t random_operands, void *stream);
+
 int ltr_abi_version(void);
 const char *ltr_strerror(int code);
 

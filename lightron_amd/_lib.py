@@ -14,7 +14,7 @@ LTR_BF16, LTR_F32 = 0, 1
 LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LTR_DKDV_BF16 = 1, 2, 4, 8, 16, 32, 64
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
-           "ltr_abi_version", "ltr_strerror")
+           "ltr_device_info", "ltr_probe_mfma", "ltr_abi_version", "ltr_strerror")
 
 _i64x3 = ctypes.c_int64 * 3
 _i64x2 = ctypes.c_int64 * 2
@@ -66,6 +66,14 @@ class RopeArgs(ctypes.Structure):
                 ("flags", ctypes.c_uint32), ("io_dtype", ctypes.c_int32)]
 
 
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [("compute_units", ctypes.c_int32), ("clock_khz", ctypes.c_int32), ("memory_clock_khz", ctypes.c_int32),
+                ("memory_bus_bits", ctypes.c_int32), ("lds_bytes_per_block", ctypes.c_int64), ("hbm_bytes", ctypes.c_int64),
+                ("arch", ctypes.c_char * 64)]
+
+
+LTR_PROBE_MIN_WORKSPACE = 8192 + 65536
+
 _lib = None
 
 
@@ -91,6 +99,10 @@ def load():
     lib.ltr_cast_f32_to_bf16.restype = ctypes.c_int
     lib.ltr_rope_apply.argtypes = [ctypes.POINTER(RopeArgs), ctypes.c_void_p]
     lib.ltr_rope_apply.restype = ctypes.c_int
+    lib.ltr_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
+    lib.ltr_device_info.restype = ctypes.c_int
+    lib.ltr_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+    lib.ltr_probe_mfma.restype = ctypes.c_int
     lib.ltr_abi_version.argtypes = []
     lib.ltr_abi_version.restype = ctypes.c_int
     lib.ltr_strerror.argtypes = [ctypes.c_int]

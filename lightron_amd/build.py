@@ -5,7 +5,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SRCS = [os.path.join(HERE, "csrc", "ltr_attn.hip"), os.path.join(HERE, "csrc", "ltr_rope.hip")]
+SRCS = [os.path.join(HERE, "csrc", f) for f in ("ltr_attn.hip", "ltr_rope.hip", "ltr_probe.hip")]
 LIB = os.path.join(HERE, "csrc", "libltr_attn.so")
 
 HIPCC_FLAGS = [
