@@ -200,12 +200,18 @@ def _device_report(la, torch, probe=True):
     for key, rnd in (("random_operands", 1), ("constant_operands", 0)):
         best = None
         for _ in range(2):      # the first launch also ramps the clock
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
             la._lib.check(lib.ltr_probe_mfma(ws.data_ptr(), n, iters, rnd, stream), "ltr_probe_mfma")
+            e1.record()
             torch.cuda.synchronize()
             t = ws[:16].view(torch.int64).cpu()
-            sec = t[0].item() / 100e6
-            cur = {"tflops": round(info.compute_units * 8 * iters * 4 * 32768.0 / sec / 1e12, 1),
-                   "shader_clock_mhz": round(t[1].item() / sec / 1e6, 0)}
+            # rate: all waves' MFMAs over the launch's duration (HIP events); clock: shader ticks against the 100 MHz wall
+            # clock over the loop of ONE wave (the two waves of a SIMD do not alternate: the older one runs its loop at the
+            # pipe's full rate, then the other; both tick counts cover the same interval, so their ratio is the clock)
+            ms = e0.elapsed_time(e1)
+            cur = {"tflops": round(info.compute_units * 8 * iters * 4 * 32768.0 / (ms * 1e-3) / 1e12, 1),
+                   "shader_clock_mhz": round(t[1].item() / (t[0].item() / 100e6) / 1e6, 0), "ms": round(ms, 3)}
             best = cur if best is None or cur["tflops"] > best["tflops"] else best
         rep["mfma_loop_" + key] = best
     return rep
@@ -333,6 +339,66 @@ def _run_attention(la, torch, cfg, steps, warmup):
             "dominant": (dom, dom_flops / (dom_ms * 1e-3) / 1e12)}
 
 
+def _run_c4_rope(la, torch, steps, warmup):
+    """Config 4's RoPE on the q side, timed both ways on the launches it touches (K is rotated beforehand in both):
+    separate passes (ltr_rope_apply on q, forward, dQ kernel, conjugate ltr_rope_apply on dQ) against the fused prologue /
+    epilogue (forward with LTR_ROPE_Q, dQ kernel with LTR_ROPE_DQ).  Also times the one-off K pass."""
+    from lightron_amd.layers import _rope_launch
+    dev = torch.device("cuda:0")
+    B, H, D, S, W = 1, 8, 128, 131072, 16
+    sl = S // W
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, sl, H, D, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(dev)
+    do = torch.randn(B, sl, H, D, generator=g).to(torch.bfloat16).to(dev)
+    table = la.rope_table(la.precompute_freqs_cis(D, S, device=dev))
+    tq = table[15 * sl:].contiguous()
+    order = [(15 - s) % W for s in range(W)]
+    k_rot = _rope_launch(k, table, False)
+    ks = [k_rot[:, j * sl:(j + 1) * sl] for j in order]
+    vs = [v[:, j * sl:(j + 1) * sl] for j in order]
+    pos = [j * sl for j in order]
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, sl, dtype=torch.float32, device=dev)
+    delta = torch.empty_like(lse)
+    dq = torch.empty_like(q)
+    q_rot = torch.empty_like(q)
+    dk = [torch.empty(0)] * W   # the dK/dV kernel is not part of this comparison
+
+    def separate():
+        qr = _rope_launch(q, tq, False)
+        la.attn_fwd(qr, ks, vs, pos, 15 * sl, None, True, out=o, lse=lse)
+        la.attn_bwd_accumulate(qr, do, lse, delta, ks, vs, pos, dq, ks, vs, 15 * sl, None, True, do_dkdv=False, o=o)
+        return _rope_launch(dq, tq, True)
+
+    def fused():
+        la.attn_fwd(q, ks, vs, pos, 15 * sl, None, True, out=o, lse=lse, q_rope=table, q_rot_out=q_rot)
+        la.attn_bwd_accumulate(q_rot, do, lse, delta, ks, vs, pos, dq, ks, vs, 15 * sl, None, True, do_dkdv=False, o=o,
+                               dq_rope=table)
+        return dq
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    t_sep, t_fus = timed(separate), timed(fused)
+    t_sep2, t_fus2 = timed(separate), timed(fused)
+    t_k = timed(lambda: _rope_launch(k, table, False))
+    return {"what": "config 4, q side: rope(q) + forward + dQ kernel + conj rope(dQ) as separate passes against the fused "
+                    "prologue / epilogue; K is rotated once beforehand in both",
+            "separate_ms": round(min(t_sep, t_sep2), 4), "fused_ms": round(min(t_fus, t_fus2), 4),
+            "k_pass_ms": round(t_k, 4)}
+
+
 def _bench_mfma_ceiling(args):
     """What the device sustains on the matrix pipe, for the record beside the attention numbers: the register-resident
     MFMA loop of ltr_probe_mfma on random and constant operands with the shader clock of each, and the vendor library's
@@ -420,6 +486,8 @@ def main():
                             "frac_of_mfma_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                             "kernel_ms": {k: v["ms_per_launch"] for k, v in r["kernels"].items()},
                             "dominant_kernel_frac": round(r["dominant"][1] / MFMA_BF16_PEAK_TFLOPS, 4)}
+        torch.cuda.empty_cache()
+        others["c4_rope"] = _run_c4_rope(la, torch, 5, 2)
         out["other_workloads"] = others
     out["device"] = _device_report(la, torch, probe=not args.no_others)
     if not args.no_cpu_baseline:

@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 4
+#define LTR_ABI_VERSION 5
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -54,6 +54,8 @@ extern "C" {
 #define LTR_DQ_BF16 16u /* backward: dq is a bf16 tensor that RECEIVES dQ of this call (no accumulation) */
 #define LTR_DELTA_FROM_O 32u /* backward: delta is computed from o by the dQ kernel (and written to delta) */
 #define LTR_DKDV_BF16 64u /* backward: chunk[c].dk / dv are bf16 tensors that RECEIVE dK / dV of this call (no accumulation) */
+#define LTR_ROPE_Q 128u   /* forward: q is un-rotated; RoPE is applied to it in the kernel's prologue (rope_freqs) */
+#define LTR_ROPE_DQ 256u  /* backward: dQ leaves the dQ kernel rotated by the conjugate angles (gradient of LTR_ROPE_Q) */
 
 /* error codes */
 #define LTR_OK 0
@@ -105,6 +107,19 @@ typedef struct ltr_attn_fwd_args {
     int32_t o_dtype;      /* LTR_BF16 or LTR_F32 */
     int32_t n_chunks;     /* 1..LTR_MAX_CHUNKS */
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
+    /* LTR_ROPE_Q (bf16 only), the fused prologue of apply_rotary_emb (layers/layers.py:44-70, applied to q at
+     * parallel/parallel_cp.py:219 and model/model.py:183): every q row is rotated, in the registers that hold it as the
+     * MFMA operand, by the angles of its GLOBAL position; no separate pass over q.  rope_freqs: the table of
+     * precompute_freqs_cis as interleaved fp32 (cos, sin), [rope_len][D/2][2], row 0 = position rope_pos0; it must
+     * cover every position of the local rows.  The rotated row has the bits ltr_rope_apply would have written.
+     * q_rot (optional, bf16, own strides): receives the rotated q, which is what ltr_attn_bwd takes as q.
+     * K is NOT rotated here: a K row is read by every q block that sees it, so its rotation belongs before the
+     * attention (one ltr_rope_apply per K tensor), not inside it. */
+    const float *rope_freqs;
+    int64_t rope_pos0;
+    int64_t rope_len;
+    void *q_rot;
+    int64_t q_rot_stride[3];
 } ltr_attn_fwd_args;
 
 int ltr_attn_fwd(const ltr_attn_fwd_args *args, void *stream);
@@ -169,13 +184,21 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;
-    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ */
     int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: scalar fp32 kernels for the 1e-4 parity cases;
                              LTR_DQ_BF16, LTR_DELTA_FROM_O and LTR_DKDV_BF16 are bf16 only and return LTR_EUNSUP with it) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];
     const void *o;        /* forward output, bf16, only read with LTR_DELTA_FROM_O */
     int64_t o_stride[3];
+    /* LTR_ROPE_DQ (bf16 only): q is the ROTATED q (q_rot of a forward with LTR_ROPE_Q); the dQ kernel's epilogue rotates
+     * dQ by the conjugate angles of each row's global position before it is stored or accumulated, so dq is the
+     * gradient of the un-rotated q (torch autograd through the complex multiply at layers/layers.py:67-70).  Table as
+     * in ltr_attn_fwd_args.  dK is the gradient of the K that was passed in (rotated beforehand: its gradient goes
+     * through ltr_rope_apply with LTR_ROPE_CONJ). */
+    const float *rope_freqs;
+    int64_t rope_pos0;
+    int64_t rope_len;
 } ltr_attn_bwd_args;
 
 int ltr_attn_bwd(const ltr_attn_bwd_args *args, void *stream);
@@ -239,8 +262,11 @@ int ltr_rope_apply(const ltr_rope_args *args, void *stream);
  * 4 * iters v_mfma_f32_32x32x16_bf16 on register-resident operands: the device's matrix-pipe ceiling.
  * random_operands != 0: the operands are read once from workspace bytes [8192, workspace_bytes), which the caller
  * fills (random bf16 data makes the chip run at the clock its power limit allows); 0: constant operands.
- * Results, valid once the stream has finished: ((int64_t *)workspace)[0] = elapsed ticks of the constant 100 MHz
- * wall clock, [1] = elapsed ticks of the shader clock counter.  Rate = CUs * 8 * iters * 4 * 32768 flop / seconds.
+ * Results, valid once the stream has finished: ((int64_t *)workspace)[0] = ticks of the constant 100 MHz wall clock
+ * that ONE wave's loop took, [1] = ticks of the shader clock counter over the same interval: their ratio is the shader
+ * clock under this load.  (The two waves of a SIMD do not alternate - the older one runs its loop at the pipe's full rate,
+ * then the other - so the rate is taken over the launch's duration, timed by the caller with events on the stream:
+ * CUs * 8 * iters * 4 * 32768 flop / seconds.)
  * workspace: device memory, 16-byte aligned, at least LTR_PROBE_MIN_WORKSPACE bytes.
  */
 typedef struct ltr_device_info_t {

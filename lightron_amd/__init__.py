@@ -3,10 +3,11 @@ from . import _lib
 from .attention import attn_fwd, attn_delta, attn_bwd_accumulate, cast_to_bf16, block_attention
 from .ring_attention import LocalRing, RingKVGrads, ring_attention_kernel, ring_attention_with_lse
 from .parallel_cp import SeqAllToAll, _all_to_all, ContextParallelAttention, LocalCPGroup
-from .layers import precompute_freqs_cis, apply_rotary_emb
+from . import layers
+from .layers import precompute_freqs_cis, apply_rotary_emb, rope_table, rope_one
 from .model import Attention, repeat_kv
 
 __all__ = ["attn_fwd", "attn_delta", "attn_bwd_accumulate", "cast_to_bf16", "block_attention",
            "LocalRing", "RingKVGrads", "ring_attention_kernel", "ring_attention_with_lse",
            "SeqAllToAll", "_all_to_all", "ContextParallelAttention", "LocalCPGroup",
-           "precompute_freqs_cis", "apply_rotary_emb", "Attention", "repeat_kv"]
+           "precompute_freqs_cis", "apply_rotary_emb", "rope_table", "rope_one", "Attention", "repeat_kv"]

@@ -7,11 +7,12 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
 
-LTR_ABI_VERSION = 4
+LTR_ABI_VERSION = 5
 LTR_MAX_CHUNKS = 32
 LTR_NOALLOC_MAX_ROWS = 1 << 20
 LTR_BF16, LTR_F32 = 0, 1
 LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LTR_DKDV_BF16 = 1, 2, 4, 8, 16, 32, 64
+LTR_ROPE_Q, LTR_ROPE_DQ = 128, 256
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_device_info", "ltr_probe_mfma", "ltr_abi_version", "ltr_strerror")
@@ -33,7 +34,9 @@ class FwdArgs(ctypes.Structure):
                 ("q_pos0", _i64x2), ("q_split", ctypes.c_int64),
                 ("scale", ctypes.c_float), ("flags", ctypes.c_uint32),
                 ("io_dtype", ctypes.c_int32), ("o_dtype", ctypes.c_int32), ("n_chunks", ctypes.c_int32),
-                ("chunk", KvChunk * LTR_MAX_CHUNKS)]
+                ("chunk", KvChunk * LTR_MAX_CHUNKS),
+                ("rope_freqs", ctypes.c_void_p), ("rope_pos0", ctypes.c_int64), ("rope_len", ctypes.c_int64),
+                ("q_rot", ctypes.c_void_p), ("q_rot_stride", _i64x3)]
 
 
 class DeltaArgs(ctypes.Structure):
@@ -55,7 +58,8 @@ class BwdArgs(ctypes.Structure):
                 ("scale", ctypes.c_float), ("flags", ctypes.c_uint32),
                 ("io_dtype", ctypes.c_int32), ("n_chunks", ctypes.c_int32),
                 ("chunk", KvChunk * LTR_MAX_CHUNKS),
-                ("o", ctypes.c_void_p), ("o_stride", _i64x3)]
+                ("o", ctypes.c_void_p), ("o_stride", _i64x3),
+                ("rope_freqs", ctypes.c_void_p), ("rope_pos0", ctypes.c_int64), ("rope_len", ctypes.c_int64)]
 
 
 class RopeArgs(ctypes.Structure):

@@ -56,6 +56,12 @@ def _norm_chunks(ks, vs):
     return _common_layout(ks), _common_layout(vs)
 
 
+def _rope_table_check(t, D, device):
+    if (t.dtype != torch.float32 or t.dim() != 3 or t.shape[1] != D // 2 or t.shape[2] != 2 or not t.is_contiguous()
+            or t.device != device):
+        raise RuntimeError("the RoPE table must be a contiguous fp32 [n_pos, D/2, 2] (cos, sin) tensor on q's device")
+
+
 def _qpos(q_pos0, Sq, q_split):
     if isinstance(q_pos0, int):
         q_pos0 = (q_pos0, q_pos0)
@@ -67,9 +73,12 @@ def _qpos(q_pos0, Sq, q_split):
 def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Tensor], k_pos0: Sequence[int],
              q_pos0=0, q_split: Optional[int] = None, causal: bool = False, scale: Optional[float] = None,
              out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None, merge: bool = False,
-             out_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+             out_dtype: Optional[torch.dtype] = None, q_rope: Optional[torch.Tensor] = None,
+             q_rot_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """One Q chunk against a table of KV chunks -> (O [B,Sq,Hq,D], LSE [B,Hq,Sq] fp32).
-    With merge=True, `out`/`lse` hold an earlier partial result which is merged in place."""
+    With merge=True, `out`/`lse` hold an earlier partial result which is merged in place.
+    q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table whose row p belongs to global position p: q is un-rotated and the
+    kernel's prologue applies RoPE to it (LTR_ROPE_Q; bf16 only); q_rot_out (bf16, like q) receives the rotated q."""
     lib = _lib.load()
     _req(q, "q")
     B, Sq, Hq, D = q.shape
@@ -98,6 +107,18 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
     a.io_dtype, a.o_dtype = _DT[q.dtype], _DT[out.dtype]
+    rope_flag = 0
+    if q_rope is not None:
+        _rope_table_check(q_rope, D, q.device)
+        a.rope_freqs, a.rope_pos0, a.rope_len = q_rope.data_ptr(), 0, q_rope.shape[0]
+        rope_flag = _lib.LTR_ROPE_Q
+        if q_rot_out is not None:
+            _req(q_rot_out, "q_rot_out")
+            if q_rot_out.dtype != torch.bfloat16 or q_rot_out.shape != q.shape:
+                raise RuntimeError("q_rot_out must be a bf16 tensor shaped like q")
+            a.q_rot, a.q_rot_stride = q_rot_out.data_ptr(), _s3(q_rot_out)
+    elif q_rot_out is not None:
+        raise RuntimeError("q_rot_out needs q_rope")
     stream = _stream_ptr(q.device)
     n = len(ks)
     with torch.cuda.device(q.device):
@@ -108,7 +129,7 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
                 ch = a.chunk[i - start]
                 ch.k, ch.v, ch.dk, ch.dv = ks[i].data_ptr(), vs[i].data_ptr(), None, None
                 ch.sk, ch.pos0 = ks[i].shape[1], int(k_pos0[i])
-            a.flags = (_lib.LTR_CAUSAL if causal else 0) | (_lib.LTR_MERGE if (merge or start > 0) else 0)
+            a.flags = (_lib.LTR_CAUSAL if causal else 0) | (_lib.LTR_MERGE if (merge or start > 0) else 0) | rope_flag
             _lib.check(lib.ltr_attn_fwd(ctypes.byref(a), stream), "ltr_attn_fwd")
     return out, lse
 
@@ -130,7 +151,7 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
-                        causal=False, scale=None, do_dq=True, do_dkdv=True, o=None, library_scratch=False):
+                        causal=False, scale=None, do_dq=True, do_dkdv=True, o=None, library_scratch=False, dq_rope=None):
     """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
     do_dq / do_dkdv select which of the two backward kernels are enqueued.  dq_acc may instead be a bf16
     tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
@@ -141,7 +162,9 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     these keys - one rank's own backward, not a ring step whose dK/dV are summed over ranks.
     library_scratch=True calls ltr_attn_bwd_noalloc instead: delta is ignored (pass None), DELTA lives in the library's
     fixed scratch array (at most LTR_NOALLOC_MAX_ROWS = B*Hq*Sq rows; calls that overlap on one GPU race on it), o is
-    required and the library allocates nothing."""
+    required and the library allocates nothing.
+    dq_rope: the (cos, sin) table of attn_fwd's q_rope; q is then the ROTATED q (q_rot_out of that forward) and the dQ
+    kernel's epilogue rotates dQ back by the conjugate angles (LTR_ROPE_DQ): dq is the gradient of the un-rotated q."""
     lib = _lib.load()
     if library_scratch and (o is None or not do_dq):
         raise RuntimeError("library_scratch needs o (DELTA is computed from it) and do_dq")
@@ -180,6 +203,12 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
                | (0 if do_dkdv else _lib.LTR_NO_DKDV) | (_lib.LTR_DQ_BF16 if dq_direct else 0)
                | (_lib.LTR_DKDV_BF16 if dkdv_direct else 0))
     a.io_dtype = _DT[q.dtype]
+    if dq_rope is not None:
+        _rope_table_check(dq_rope, D, q.device)
+        if not do_dq:
+            raise RuntimeError("dq_rope rotates dQ in the dQ kernel's epilogue: do_dq must be set")
+        a.rope_freqs, a.rope_pos0, a.rope_len = dq_rope.data_ptr(), 0, dq_rope.shape[0]
+        a.flags |= _lib.LTR_ROPE_DQ
     if o is not None:
         if not do_dq:
             raise RuntimeError("delta from o is computed by the dQ kernel: do_dq must be set")
@@ -222,19 +251,24 @@ class BlockAttentionFunction(torch.autograd.Function):
     fixed arguments are k_0..k_{n-1}, v_0..v_{n-1}."""
 
     @staticmethod
-    def forward(ctx, q, n_chunks, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, kv_grad_acc, *kv):
+    def forward(ctx, q, n_chunks, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, kv_grad_acc, q_rope, *kv):
         ks, vs = list(kv[:n_chunks]), list(kv[n_chunks:])
+        # fused RoPE prologue: the kernel rotates q on load and hands the rotated q back for the backward
+        q_rot = torch.empty(q.shape, dtype=q.dtype, device=q.device) if q_rope is not None else None
         if stepwise:
             # one launch per KV chunk, merged in the epilogue into an fp32 running (O, LSE)
-            o, lse = attn_fwd(q, ks[:1], vs[:1], k_pos0[:1], q_pos0, q_split, causal, scale, out_dtype=torch.float32)
+            o, lse = attn_fwd(q, ks[:1], vs[:1], k_pos0[:1], q_pos0, q_split, causal, scale, out_dtype=torch.float32,
+                              q_rope=q_rope, q_rot_out=q_rot)
             for i in range(1, n_chunks):
                 attn_fwd(q, ks[i:i + 1], vs[i:i + 1], k_pos0[i:i + 1], q_pos0, q_split, causal, scale,
-                         out=o, lse=lse, merge=True)
+                         out=o, lse=lse, merge=True, q_rope=q_rope)
             if (out_dtype or q.dtype) != torch.float32:
                 o = o.to(out_dtype or q.dtype)
         else:
-            o, lse = attn_fwd(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, out_dtype=out_dtype)
-        ctx.save_for_backward(q, o, lse, *kv)
+            o, lse = attn_fwd(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, out_dtype=out_dtype,
+                              q_rope=q_rope, q_rot_out=q_rot)
+        ctx.q_rope = q_rope
+        ctx.save_for_backward(q if q_rot is None else q_rot, o, lse, *kv)
         ctx.meta = (n_chunks, list(k_pos0), q_pos0, q_split, causal, scale)
         ctx.kv_grad_acc = kv_grad_acc
         ctx.mark_non_differentiable(lse)
@@ -265,9 +299,9 @@ class BlockAttentionFunction(torch.autograd.Function):
             # accumulators and cast once at the end, instead of one bf16 rounding per node: nothing flows to k, v here
             dk_accs, dv_accs = ctx.kv_grad_acc
             attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal,
-                                scale, o=o if fuse else None)
+                                scale, o=o if fuse else None, dq_rope=ctx.q_rope)
             dq = dq_acc if (direct or f32) else cast_to_bf16(dq_acc)
-            return (dq, None, None, None, None, None, None, None, None, None) + (None,) * (2 * n_chunks)
+            return (dq, None, None, None, None, None, None, None, None, None, None) + (None,) * (2 * n_chunks)
         lens = [k.shape[1] for k in ks]
         shape = (ks[0].shape[0], sum(lens), ks[0].shape[2], ks[0].shape[3])
         if f32:
@@ -280,17 +314,20 @@ class BlockAttentionFunction(torch.autograd.Function):
         dk_accs = [dk_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         dv_accs = [dv_buf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0, q_split, causal, scale,
-                            o=o if fuse else None)
+                            o=o if fuse else None, dq_rope=ctx.q_rope)
         dq = dq_acc if (direct or f32) else cast_to_bf16(dq_acc)
         dk16, dv16 = dk_buf, dv_buf
         dks = [dk16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
         dvs = [dv16[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
-        return (dq, None, None, None, None, None, None, None, None, None, *dks, *dvs)
+        return (dq, None, None, None, None, None, None, None, None, None, None, *dks, *dvs)
 
 
 def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, scale=None, stepwise=False,
-                    out_dtype=None, kv_grad_acc=None):
-    """Differentiable entry: returns (O, LSE).  kv_grad_acc = (dk_accs, dv_accs), fp32 tensors shaped like ks / vs:
+                    out_dtype=None, kv_grad_acc=None, q_rope=None):
+    """Differentiable entry: returns (O, LSE).  q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table indexed by global
+    position (layers.rope_table of precompute_freqs_cis): q is un-rotated, the forward kernel's prologue applies RoPE
+    to it and the dQ kernel's epilogue the conjugate rotation, so no separate pass touches q or dQ (bf16 only).  ks are
+    taken as given: rotate K once beforehand (apply_rotary_emb), it is read by every q block.  kv_grad_acc = (dk_accs, dv_accs), fp32 tensors shaped like ks / vs:
     the backward then ADDS dK / dV into them (no gradient flows to ks / vs through autograd); the owner of the
     accumulators makes the one final cast.  That is how a ring sums dK / dV over its ranks without a bf16 rounding
     per rank."""
@@ -302,5 +339,7 @@ def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, sca
         for a, k in zip(list(dk_accs) + list(dv_accs), list(ks) + list(vs)):
             if a.dtype != torch.float32 or a.shape != k.shape:
                 raise RuntimeError("kv_grad_acc entries must be fp32 tensors shaped like their chunks")
+    if q_rope is not None and q.dtype != torch.bfloat16:
+        raise RuntimeError("the fused RoPE prologue is implemented for bf16 q")
     return BlockAttentionFunction.apply(q, n, list(k_pos0), q_pos0, q_split, causal, scale, stepwise, out_dtype,
-                                        kv_grad_acc, *ks, *vs)
+                                        kv_grad_acc, q_rope, *ks, *vs)

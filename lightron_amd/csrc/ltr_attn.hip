@@ -74,6 +74,10 @@ struct FwdParams {
     unsigned flags;
     int o_f32;
     int n_chunks;
+    const float *rope;     // LTR_ROPE_Q: (cos, sin) rows, D floats per position, row 0 = position rope_pos0
+    int rope_pos0;
+    void *q_rot;           // optional bf16 output: the rotated q
+    long long qrs[3];
     ChunkDev chunk[LTR_MAX_CHUNKS];
 };
 
@@ -94,6 +98,8 @@ struct BwdParams {
     unsigned flags;
     int n_chunks;
     int tiles_total;  // key tiles over all chunks
+    const float *rope;     // LTR_ROPE_DQ: (cos, sin) rows, D floats per position, row 0 = position rope_pos0
+    int rope_pos0;
     ChunkDev chunk[LTR_MAX_CHUNKS];
 };
 
@@ -208,6 +214,38 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) {
     union { uint4 u; bf16x8 v; } c;
     c.u = x;
     return c.v;
+}
+
+// Rotary position embedding of 8 consecutive elements (4 adjacent (re, im) pairs) of one row: f0, f1 hold the pairs'
+// (cos, sin).  The arithmetic of apply_rotary_emb (layers/layers.py:44-70) as the streaming kernel of ltr_rope_apply does
+// it: fp32 complex multiply with the four products rounded separately, result rounded to bf16 - so a row rotated here has
+// the bits that the separate pass would have written.
+__device__ __forceinline__ bf16x8 rope_rotate8(bf16x8 x, f32x4 f0, f32x4 f1) {
+#pragma clang fp contract(off)
+    const float cs[4] = {f0[0], f0[2], f1[0], f1[2]}, sn[4] = {f0[1], f0[3], f1[1], f1[3]};
+    bf16x8 out;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float re = (float)x[2 * i], im = (float)x[2 * i + 1];
+        const float rr = re * cs[i], ii = im * sn[i];
+        const float ri = re * sn[i], ir = im * cs[i];
+        out[2 * i] = (__bf16)(rr - ii);
+        out[2 * i + 1] = (__bf16)(ri + ir);
+    }
+    return out;
+}
+
+// Gradient of that rotation: 4 consecutive fp32 elements (2 pairs) times the CONJUGATE angles; f = (cos, sin, cos, sin).
+__device__ __forceinline__ f32x4 rope_conj4(f32x4 v, f32x4 f) {
+#pragma clang fp contract(off)
+    f32x4 out;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float re = v[2 * i], im = v[2 * i + 1], c = f[2 * i], sn = f[2 * i + 1];
+        out[2 * i] = re * c + im * sn;
+        out[2 * i + 1] = im * c - re * sn;
+    }
+    return out;
 }
 
 struct PackedTile {   // 16 bf16 values of one lane's 32x32 tile column, as the two B operands of K = 16
@@ -465,6 +503,17 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             uint4 x = make_uint4(0, 0, 0, 0);
             if (row_ok) x = *(const uint4 *)(qp + kb * 16 + 8 * hh);
             qreg[kb] = as_bf16x8(x);
+        }
+        // fused RoPE prologue: q arrives un-rotated and is rotated here, in the registers that hold it as the MFMA operand,
+        // by the angles of the row's global position; the rotated row can be stored for the backward
+        if ((p.flags & LTR_ROPE_Q) && row_ok) {
+            const float *fr = p.rope + (long long)(my_pos - p.rope_pos0) * D + 8 * hh;
+            __bf16 *qr = p.q_rot ? (__bf16 *)p.q_rot + b * p.qrs[0] + (long long)my_row * p.qrs[1] + h * p.qrs[2] + 8 * hh : nullptr;
+#pragma unroll
+            for (int kb = 0; kb < D / 16; kb++) {
+                qreg[kb] = rope_rotate8(qreg[kb], *(const f32x4 *)(fr + 16 * kb), *(const f32x4 *)(fr + 16 * kb + 4));
+                if (qr) *(bf16x8 *)(qr + 16 * kb) = qreg[kb];
+            }
         }
     }
 
@@ -1563,10 +1612,21 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
         const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + w * 32);
         const long long dqs1 = uniform64(p.dqs[1]);
         const long long off0 = uniform64(b * p.dqs[0] + h * p.dqs[2]) + (wave_row0 + lane / LPR) * dqs1 + 4 * (lane % LPR);
+        // LTR_ROPE_DQ: q was rotated by the forward's prologue, so the gradient of the caller's un-rotated q is dQ rotated by
+        // the conjugate angles of its row's position (the rotation is linear: it commutes with the accumulation over calls)
+        const bool rope = uniform32(p.flags & LTR_ROPE_DQ) != 0;
+        const float *const rope_tab = p.rope;
+        const int rope_p0 = uniform32(p.rope_pos0), split_u = uniform32(p.q_split), qp0 = uniform32(p.q_pos0[0]), qp1 = uniform32(p.q_pos0[1]);
+        auto unrotate = [&](int row, int col, f32x4 val) {
+            if (!rope) return val;
+            const int pos = q_position(wave_row0 + row, split_u, qp0, qp1);
+            return rope_conj4(val, *(const f32x4 *)(rope_tab + (long long)(pos - rope_p0) * D + col));
+        };
         if (uniform32(p.flags & LTR_DQ_BF16)) {   // this call saw every key of these rows: store the result, no accumulator
             __bf16 *dqp = (__bf16 *)p.dq + off0;
-            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int, f32x4 val) {
+            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int col, f32x4 val) {
                 if (wave_row0 + row < Sq_u) {
+                    val = unrotate(row, col, val);
                     bf16x4 y;
 #pragma unroll
                     for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
@@ -1584,8 +1644,9 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
                 if (wave_row0 + it * ROWS_PER_IT + lane / LPR < Sq_u) old[it] = *(const f32x4 *)(dqp + it * ROWS_PER_IT * dqs1);
             }
             int it = 0;
-            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int, f32x4 val) {
+            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int col, f32x4 val) {
                 if (wave_row0 + row < Sq_u) {
+                    val = unrotate(row, col, val);
 #pragma unroll
                     for (int e = 0; e < 4; e++) val[e] += old[it][e];
                     *(f32x4 *)dqp = val;
@@ -1871,6 +1932,14 @@ bool strides_ok(const int64_t *s, int elem_bytes) {
 
 int fits_i32(int64_t x) { return x >= 0 && x < (int64_t)0x7fffffff; }
 
+// every position of the local rows lies inside the rows [pos0, pos0 + len) of a RoPE table
+bool rope_table_covers(const int64_t *q_pos0, int64_t q_split, int64_t Sq, int64_t pos0, int64_t len) {
+    if (len <= 0 || !fits_i32(pos0)) return false;
+    if (q_split > 0 && (q_pos0[0] < pos0 || q_pos0[0] + q_split > pos0 + len)) return false;
+    if (Sq > q_split && (q_pos0[1] < pos0 || q_pos0[1] + (Sq - q_split) > pos0 + len)) return false;
+    return true;
+}
+
 // ------------------------------------------------------------------------------ fixed scratch
 // DELTA workspace of ltr_attn_bwd_noalloc: a fixed array in device memory that belongs to the library (every device the
 // library runs on holds its own copy until the process ends).  Host code never uses the array's name as an address: the
@@ -1918,7 +1987,7 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     if (!a || !a->q || !a->o || !a->lse) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE)) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     if (a->o_dtype != LTR_BF16 && a->o_dtype != LTR_F32) return LTR_EUNSUP;
@@ -1932,6 +2001,20 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     for (int i = 0; i < 3; i++)
         if (a->o_stride[i] < 0 || (a->o_stride[i] * ob) % 8) return LTR_EALIGN;
     FwdParams p;
+    p.rope = nullptr;
+    p.rope_pos0 = 0;
+    p.q_rot = nullptr;
+    for (int i = 0; i < 3; i++) p.qrs[i] = 0;
+    if (a->flags & LTR_ROPE_Q) {
+        if (a->io_dtype != LTR_BF16) return LTR_EUNSUP;
+        if (!a->rope_freqs) return LTR_EINVAL;
+        if (!rope_table_covers(a->q_pos0, a->q_split, a->Sq, a->rope_pos0, a->rope_len)) return LTR_EINVAL;
+        if (!aligned16(a->rope_freqs) || (a->q_rot && (!aligned16(a->q_rot) || !strides_ok(a->q_rot_stride, 2)))) return LTR_EALIGN;
+        p.rope = a->rope_freqs;
+        p.rope_pos0 = (int)a->rope_pos0;
+        p.q_rot = a->q_rot;
+        for (int i = 0; i < 3; i++) p.qrs[i] = a->q_rot ? a->q_rot_stride[i] : 0;
+    }
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];
         if (!ch.k || !ch.v || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
@@ -2028,13 +2111,13 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16)) return LTR_EINVAL;
+    if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ)) return LTR_EINVAL;
     const bool fused_delta = flags & LTR_DELTA_FROM_O;
     if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     const bool f32 = a->io_dtype == LTR_F32;
-    if (f32 && (flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16))) return LTR_EUNSUP;   // bf16 conveniences only
+    if (f32 && (flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ))) return LTR_EUNSUP;   // bf16 conveniences only
     const int gb = (flags & LTR_DKDV_BF16) ? 2 : 4;   // bytes per dK / dV element
     const int eb = f32 ? 4 : 2;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
@@ -2051,6 +2134,15 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     if ((a->Sq + 63) / 64 > BwdLds<128>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
     if ((a->Sq + 64) * a->q_stride[1] >= 0x7fffffffLL || (a->Sq + 64) * a->do_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     BwdParams p;
+    p.rope = nullptr;
+    p.rope_pos0 = 0;
+    if (flags & LTR_ROPE_DQ) {
+        if (!do_dq || !a->rope_freqs) return LTR_EINVAL;
+        if (!rope_table_covers(a->q_pos0, a->q_split, a->Sq, a->rope_pos0, a->rope_len)) return LTR_EINVAL;
+        if (!aligned16(a->rope_freqs)) return LTR_EALIGN;
+        p.rope = a->rope_freqs;
+        p.rope_pos0 = (int)a->rope_pos0;
+    }
     long long tiles = 0;
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];

@@ -4,7 +4,8 @@
 //                       stay in registers (no memory traffic inside the loop): the matrix pipe is the only limit.  With
 //                       operands taken from the caller's workspace (random data) the chip runs at the clock its power
 //                       limit allows; with constant operands it toggles few bits and keeps a higher clock.
-//   Block 0 reports the elapsed ticks of the constant 100 MHz wall clock and of the shader clock counter.
+//   The first wave of block 0 reports the ticks of the constant 100 MHz wall clock and of the shader clock counter over its own
+//   loop (their ratio is the shader clock under this load); the rate is taken by the caller over the whole launch.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "ltr_attn.h"

@@ -1,6 +1,7 @@
-"""RoPE with the reference's conventions (layers/layers.py:18-70).  On GPU tensors the rotation is one
-streaming HIP kernel (ltr_rope_apply) with the conjugate rotation as its gradient; the angle table is
-built with torch ops exactly as the reference builds it."""
+"""RoPE with the reference's conventions (layers/layers.py:18-70).  The rotation is one streaming HIP kernel
+(ltr_rope_apply) with the conjugate rotation as its gradient - or, for q, the prologue of the attention kernel itself
+(block_attention(..., q_rope=rope_table(freqs_cis))); the angle table is built with torch ops exactly as the reference
+builds it."""
 import ctypes
 
 import torch
@@ -57,6 +58,16 @@ class _Rope(torch.autograd.Function):
         return _rope_launch(grad, table, True), None
 
 
+def rope_table(freqs_cis: torch.Tensor, device=None) -> torch.Tensor:
+    """The complex64 table of precompute_freqs_cis as the fp32 [S, D/2, 2] (cos, sin) rows the HIP kernels read."""
+    return torch.view_as_real(freqs_cis.to(device=device or freqs_cis.device, dtype=torch.complex64)).contiguous()
+
+
+def rope_one(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
+    """apply_rotary_emb for ONE GPU tensor (K, when q's rotation is fused into the attention kernel)."""
+    return _rope_gpu(x, freqs_cis)
+
+
 def _rope_gpu(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
     if x.dtype not in (torch.bfloat16, torch.float32):
         raise TypeError("apply_rotary_emb on the GPU takes bf16 or fp32 tensors, got %s" % x.dtype)
@@ -70,16 +81,8 @@ def _rope_gpu(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
 
 
 def apply_rotary_emb(xq, xk, freqs_cis):
-    """Rotate adjacent pairs (x[2i], x[2i+1]) in fp32 and cast back (layers.py:44-70).
-    GPU tensors go through the HIP kernel (and only through it); tensors that live on the host are
-    rotated with the reference's own torch formulation."""
-    if xq.is_cuda != xk.is_cuda:
-        raise ValueError("xq and xk must live on the same kind of device")
-    if xq.is_cuda:
-        return _rope_gpu(xq, freqs_cis), _rope_gpu(xk, freqs_cis)
-    xq_ = torch.view_as_complex(xq.float().reshape(*xq.shape[:-1], -1, 2))
-    xk_ = torch.view_as_complex(xk.float().reshape(*xk.shape[:-1], -1, 2))
-    fc = reshape_for_broadcast(freqs_cis, xq_)
-    xq_out = torch.view_as_real(xq_ * fc).flatten(3)
-    xk_out = torch.view_as_real(xk_ * fc).flatten(3)
-    return xq_out.type_as(xq), xk_out.type_as(xk)
+    """Rotate adjacent pairs (x[2i], x[2i+1]) in fp32 and cast back (layers.py:44-70), on the GPU through the HIP
+    kernel and only through it: tensors that live on the host are refused, like everywhere else in this package."""
+    if not (xq.is_cuda and xk.is_cuda):
+        raise RuntimeError("apply_rotary_emb takes GPU tensors (the HIP library has no CPU path)")
+    return _rope_gpu(xq, freqs_cis), _rope_gpu(xk, freqs_cis)

@@ -9,7 +9,7 @@ import torch
 from torch import nn
 
 from .attention import block_attention
-from .layers import apply_rotary_emb
+from .layers import apply_rotary_emb, rope_one, rope_table
 
 
 def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
@@ -44,7 +44,15 @@ class Attention(nn.Module):
         xq = self.wq(x).view(B, S, self.n_heads, self.head_dim)
         xk = self.wk(x).view(B, S, self.n_kv_heads, self.head_dim)
         xv = self.wv(x).view(B, S, self.n_kv_heads, self.head_dim)
-        xq, xk = apply_rotary_emb(xq, xk, freqs_cis)                  # model.py:183, before any head repetition
+        # RoPE (model.py:183, before any head repetition): K in one streaming pass; q inside the attention kernel, whose
+        # prologue rotates each row in registers (and whose dQ epilogue rotates the gradient back) when q is bf16
         # causal attention, scale 1/sqrt(D), [B, S, H, D] in and out: no transposes, no repeat_kv copy
-        out, _ = block_attention(xq, [xk], [xv], [0], 0, None, causal=True)
+        if xq.dtype == torch.bfloat16:
+            if freqs_cis.shape != (S, self.head_dim // 2):               # layers.py:34
+                raise AssertionError("freqs_cis shape %s does not match x shape %s" % (tuple(freqs_cis.shape), (S, self.head_dim // 2)))
+            xk = rope_one(xk, freqs_cis)
+            out, _ = block_attention(xq, [xk], [xv], [0], 0, None, causal=True, q_rope=rope_table(freqs_cis, xq.device))
+        else:
+            xq, xk = apply_rotary_emb(xq, xk, freqs_cis)
+            out, _ = block_attention(xq, [xk], [xv], [0], 0, None, causal=True)
         return self.wo(out.reshape(B, S, -1))

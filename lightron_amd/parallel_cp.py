@@ -14,7 +14,7 @@ import torch
 import torch.nn as nn
 
 from .attention import block_attention
-from .layers import apply_rotary_emb
+from .layers import apply_rotary_emb, rope_one, rope_table
 
 
 class LocalCPGroup:
@@ -136,18 +136,22 @@ class ContextParallelAttention(nn.Module):
             o = o.view(W, B, S_global, H // W, D)
             o = _all_to_all(o, 1, 2, self.cp_group)              # [W, B, S_local, H, D]
         else:
+            # RoPE at global positions (:215-219): every K shard is rotated once, in one streaming pass (it is read by
+            # every later q shard); q is rotated inside the attention kernel's prologue, dQ rotated back in the dQ
+            # kernel's epilogue (bf16; fp32 inputs take the streaming pass for q as well)
             outs = []
+            fused = xq.dtype == torch.bfloat16
+            table = rope_table(fc, xq.device) if fused else None
             qs, ks = [], []
             for j in range(W):
                 fj = fc[j * S_local:(j + 1) * S_local]
-                qj, kj = apply_rotary_emb(xq[j], xk[j], fj) if H == Hkv else _rope_each(xq[j], xk[j], fj)
-                qs.append(qj)
-                ks.append(kj)
+                ks.append(rope_one(xk[j], fj))
+                qs.append(xq[j] if fused else rope_one(xq[j], fj))
             vs = [xv[j] for j in range(W)]
             pos = [j * S_local for j in range(W)]
             for j in range(W):
                 n = j + 1 if self.causal else W                  # later shards are fully masked
-                oj, _ = block_attention(qs[j], ks[:n], vs[:n], pos[:n], j * S_local, None, self.causal)
+                oj, _ = block_attention(qs[j], ks[:n], vs[:n], pos[:n], j * S_local, None, self.causal, q_rope=table)
                 outs.append(oj)
             o = torch.stack(outs, 0)
         return self.local_attn.wo(o.flatten(3))

@@ -161,11 +161,14 @@ def test_config3_full_ring_entry_point_fp32_kv_grads(ltr):
     assert _rel(dv.double().sum(1), rhs) < 1e-2
 
 
-@pytest.mark.parametrize("path", ["accumulators", "bench"])
+@pytest.mark.parametrize("path", ["accumulators", "bench", "fused_rope"])
 def test_config4_full_rank15(ltr, path):
     """B=1, H=8, D=128, S=131072 as 16 chunks of 8192, bf16, causal, RoPE (base 10000) applied to
     q and k beforehand; rank 15's Q chunk against all 16 KV chunks: O, LSE, dQ and this rank's
-    contribution to dK, dV of every chunk.  The two paths are those of test_config3_full_all_ranks."""
+    contribution to dK, dV of every chunk.  Paths "accumulators" and "bench" are those of test_config3_full_all_ranks;
+    "fused_rope" hands the kernels the UN-rotated q chunk: the forward's prologue rotates it (positions 122880 ..
+    131071; the rotated q must have the bits of the separate pass), the dQ kernel's epilogue rotates dQ back, and dQ is
+    compared with the oracle's dQ of the rotated q carried through the conjugate rotation."""
     g = torch.Generator().manual_seed(0)
     B, H, D, S, W = 1, 8, 128, 131072, 16
     sl = S // W
@@ -180,6 +183,7 @@ def test_config4_full_rank15(ltr, path):
     fc_gpu = ltr.precompute_freqs_cis(D, S, device="cuda").cpu()
     assert torch.equal(ltr.precompute_freqs_cis(D, S), fc_cpu) or (ltr.precompute_freqs_cis(D, S) - fc_cpu).abs().max() < 1e-6
     assert (torch.angle(fc_gpu * fc_cpu.conj())).abs().max() < 3e-2
+    q_raw = q
     qd, kd = ltr.apply_rotary_emb(q.cuda(), k.cuda(), fc)
     vd = v.cuda()
     q, k = qd.cpu(), kd.cpu()                                              # the oracle sees the rotated bf16 inputs
@@ -189,20 +193,32 @@ def test_config4_full_rank15(ltr, path):
     ro_q, _ = orc.apply_rotary_emb(x, x, fc_cpu[S - 64:])
     rg_q, _ = ltr.apply_rotary_emb(x.cuda(), x.cuda(), fc[S - 64:])
     assert (rg_q.cpu() - ro_q).abs().max() < 1e-5, (rg_q.cpu() - ro_q).abs().max()
+    q_unrot = q_raw[:, 15 * sl:].cuda() if path == "fused_rope" else None
     ql, dol = qd[:, 15 * sl:].contiguous(), do.cuda()
     ks = [kd[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
     vs = [vd[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
     pos0 = [j * sl for j in orc.ring_order(15, W)]
-    ol, lsel = ltr.attn_fwd(ql, ks, vs, pos0, 15 * sl, None, True)
+    if path == "fused_rope":
+        table = ltr.rope_table(fc)
+        q_rot = torch.empty_like(ql)
+        ol, lsel = ltr.attn_fwd(q_unrot, ks, vs, pos0, 15 * sl, None, True, q_rope=table, q_rot_out=q_rot)
+        assert torch.equal(q_rot, ql)
+    else:
+        ol, lsel = ltr.attn_fwd(ql, ks, vs, pos0, 15 * sl, None, True)
     dk = torch.zeros(kd.shape, dtype=torch.float32, device="cuda")
     dv = torch.zeros(vd.shape, dtype=torch.float32, device="cuda")
     dks = [dk[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
     dvs = [dv[:, j * sl:(j + 1) * sl] for j in orc.ring_order(15, W)]
-    if path == "bench":
+    if path in ("bench", "fused_rope"):
         dq = torch.empty(ql.shape, dtype=torch.bfloat16, device="cuda")
         delta_ws = torch.empty(B, H, sl, dtype=torch.float32, device="cuda")
-        ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True, do_dkdv=False, o=ol)
+        ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True, do_dkdv=False, o=ol,
+                                dq_rope=table if path == "fused_rope" else None)
         ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, 15 * sl, None, True, do_dq=False)
+        if path == "fused_rope":
+            # dq is the gradient of the un-rotated q; rotating it forward again gives the gradient of the rotated q (the
+            # rotation is orthogonal), which is what the sampled-row check below computes
+            dq = ltr.rope_one(dq, fc[15 * sl:])
     else:
         delta = ltr.attn_delta(ol, dol)
         dq = torch.zeros(ql.shape, dtype=torch.float32, device="cuda")

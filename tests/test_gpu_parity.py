@@ -753,6 +753,80 @@ def test_more_chunks_than_one_launch_holds(ltr, dtype, n_chunks):
     assert dk[:, q_pos0 + Sq:].abs().max() == 0 and dv[:, q_pos0 + Sq:].abs().max() == 0    # keys no query sees
 
 
+@pytest.mark.parametrize("D,Hq,Hkv,Sq,q_pos,chunks,causal", [
+    (128, 4, 2, 300, (1000, 1000), [(700, 400), (1100, 200)], True),      # contiguous rows, two KV chunks
+    (64, 4, 4, 256, (0, 768), [(0, 512), (512, 512)], True),              # zig-zag rows (two segments), D = 64
+    (128, 2, 1, 77, (130000, 130000), [(129900, 250)], False),            # positions near the top of a 131072 table
+])
+def test_fused_rope_prologue_and_dq_epilogue(ltr, D, Hq, Hkv, Sq, q_pos, chunks, causal):
+    """LTR_ROPE_Q / LTR_ROPE_DQ against the separate pass (ltr_rope_apply on q, attention, conjugate ltr_rope_apply on
+    dQ) and against the oracle (apply_rotary_emb restated, then dense attention and its autograd).  The rotated q and
+    therefore O and LSE must have the SAME BITS as with the separate pass; dQ is rounded once instead of twice, so it is
+    compared with a tolerance (and must not be further from the oracle than the two-pass result)."""
+    g = torch.Generator().manual_seed(31 + Sq)
+    B = 2
+    n_pos = max(max(p0 + n for p0, n in chunks), max(q_pos) + Sq) + 5
+    fc = orc.precompute_freqs_cis(D, n_pos)
+    split = Sq // 2 if q_pos[0] != q_pos[1] else Sq
+    qpos = torch.cat([torch.arange(split) + q_pos[0], torch.arange(Sq - split) + q_pos[1]])
+    q, do = _randn((B, Sq, Hq, D), g, torch.bfloat16), _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    ks = [_randn((B, n, Hkv, D), g, torch.bfloat16) for _, n in chunks]
+    vs = [_randn((B, n, Hkv, D), g, torch.bfloat16) for _, n in chunks]
+    kpos = torch.cat([torch.arange(n) + p0 for p0, n in chunks])
+    # oracle: rotate (fp32 complex multiply, cast back to bf16 as the reference does), dense attention, autograd
+    q_rot_ref, _ = orc.apply_rotary_emb(q, q, fc[qpos])
+    k_rot = [orc.apply_rotary_emb(k, k, fc[p0:p0 + n])[0] for k, (p0, n) in zip(ks, chunks)]
+    o_ref, lse_ref, dq_rot_ref, _, _ = orc.dense_attention_grads(q_rot_ref.float(), torch.cat(k_rot, 1).float(), torch.cat(vs, 1).float(),
+                                                                 do.float(), qpos, kpos, causal)
+    conj = torch.conj(fc[qpos])
+    dq_ref = torch.view_as_real(torch.view_as_complex(dq_rot_ref.float().reshape(B, Sq, Hq, D // 2, 2)) * conj[None, :, None, :]).flatten(3)
+
+    fcd = fc.cuda()
+    table = ltr.rope_table(fcd)
+    kd = [ltr.rope_one(k.cuda(), fcd[p0:p0 + n]) for k, (p0, n) in zip(ks, chunks)]
+    for a, b in zip(kd, k_rot):
+        assert torch.equal(a.cpu(), b)
+    vd = [v.cuda() for v in vs]
+    pos0 = [p0 for p0, _ in chunks]
+    qd = q.cuda()
+    # separate pass
+    q_rot_2p = ltr.rope_one(qd, fcd[qpos.cuda()])
+    assert torch.equal(q_rot_2p.cpu(), q_rot_ref)
+    o2, lse2 = ltr.attn_fwd(q_rot_2p, kd, vd, pos0, q_pos, split, causal)
+    # fused prologue
+    q_rot = torch.full_like(qd, float("nan"))
+    o1, lse1 = ltr.attn_fwd(qd, kd, vd, pos0, q_pos, split, causal, q_rope=table, q_rot_out=q_rot)
+    assert torch.equal(q_rot, q_rot_2p)
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+    assert (o1.cpu().double() - o_ref).abs().max() < O_TOL_BF16
+    fin = torch.isfinite(lse_ref)
+    assert (lse1.cpu().double()[fin] - lse_ref[fin]).abs().max() < LSE_TOL_BF16
+
+    # through autograd: fused (q un-rotated in, gradient of un-rotated q out) and two-pass
+    def grads(fused):
+        qg = qd.clone().requires_grad_(True)
+        if fused:
+            o, _ = ltr.block_attention(qg, kd, vd, pos0, q_pos, split, causal, q_rope=table)
+        else:
+            o, _ = ltr.block_attention(ltr.rope_one(qg, fcd[qpos.cuda()]), kd, vd, pos0, q_pos, split, causal)
+        o.backward(do.cuda())
+        return qg.grad.cpu()
+    dq_f, dq_2 = grads(True), grads(False)
+    e_f, e_2 = _rel(dq_f, dq_ref), _rel(dq_2, dq_ref)
+    assert e_f < GRAD_RTOL_BF16 and e_2 < GRAD_RTOL_BF16, (e_f, e_2)
+    assert e_f <= e_2 * 1.05 + 1e-4, (e_f, e_2)                     # one rounding instead of two
+    assert _rel(dq_f, dq_2.double()) < 1e-2
+    # the fp32 accumulator form of the dQ epilogue (two launches' worth of chunks accumulate rotated partials)
+    delta = ltr.attn_delta(o1, do.cuda())
+    acc = torch.zeros(qd.shape, dtype=torch.float32, device="cuda")
+    dk = [torch.zeros(k.shape, dtype=torch.float32, device="cuda") for k in kd]
+    dv = [torch.zeros(k.shape, dtype=torch.float32, device="cuda") for k in kd]
+    for i in range(len(kd)):
+        ltr.attn_bwd_accumulate(q_rot, do.cuda(), lse1, delta, kd[i:i + 1], vd[i:i + 1], pos0[i:i + 1], acc, dk[i:i + 1], dv[i:i + 1],
+                                q_pos, split, causal, do_dkdv=False, dq_rope=table)
+    assert _rel(acc.cpu(), dq_ref) < GRAD_RTOL_BF16
+
+
 @pytest.mark.parametrize("seed", list(range(8)))
 def test_rope_sweep_bit_exact(ltr, seed):
     """ltr_rope_apply on random shapes, dtypes, layouts and starting positions against the oracle, bit for bit."""
