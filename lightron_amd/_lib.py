@@ -5,7 +5,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "csrc", "libltr_attn.so")
+# LTR_ATTN_LIB names another build of the same library (same ABI version), e.g. to compare two builds in one session
+LIB_PATH = os.environ.get("LTR_ATTN_LIB") or os.path.join(HERE, "csrc", "libltr_attn.so")
 
 LTR_ABI_VERSION = 5
 LTR_MAX_CHUNKS = 32

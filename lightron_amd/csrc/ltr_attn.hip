@@ -37,6 +37,7 @@
 #include <math.h>
 #include <type_traits>
 #include <atomic>
+#include <algorithm>
 #include "ltr_attn.h"
 
 namespace {
@@ -2222,12 +2223,19 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     const long long nblk_q = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
     if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
     // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
-    if (a->D == 128) {
-        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
-        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
-    } else {
-        if (do_dq) hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
-        if (do_dkdv) hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
+    if (do_dq) {
+        if (a->D == 128) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
+        else hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
+    }
+    if (do_dkdv) {
+        // A block of the dK/dV kernel owns 128 keys and loops over the query tiles that see them: under a causal mask its
+        // work falls with the keys' position.  The blocks of one (batch, kv head) are handed out in the order of the chunk
+        // table, so the table of THIS kernel is sorted by position: the longest blocks start first and the short ones fill
+        // the tail (the sums inside a block do not depend on the table's order).
+        if (flags & LTR_CAUSAL)
+            std::stable_sort(p.chunk, p.chunk + p.n_chunks, [](const ChunkDev &x, const ChunkDev &y) { return x.pos0 < y.pos0; });
+        if (a->D == 128) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
+        else hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
