@@ -68,6 +68,7 @@ struct FwdParams {
     float *lse;
     int B, Hq, Hkv, n_rep;
     int Sq, n_qtiles;
+    int n_slots;           // q tiles are handed out in slots: n_qtiles of one tile, or (n_qtiles + 1) / 2 of two (see q_tile_slots)
     long long qs[3], os[3], ks[3], vs[3];
     int q_pos0[2];
     int q_split;
@@ -99,6 +100,7 @@ struct BwdParams {
     unsigned flags;
     int n_chunks;
     int tiles_total;  // key tiles over all chunks
+    int n_slots;      // slots of 256-row q tiles of the dQ kernel (see q_tile_slots)
     const float *rope;     // LTR_ROPE_DQ: (cos, sin) rows, D floats per position, row 0 = position rope_pos0
     int rope_pos0;
     ChunkDev chunk[LTR_MAX_CHUNKS];
@@ -472,16 +474,28 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     int idx = blockIdx.x, pair, rest;
     const int P = p.B * p.Hkv;
     if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3, nr = p.n_qtiles * p.n_rep;
+        int xcd = idx & 7, j = idx >> 3, nr = p.n_slots * p.n_rep;
         pair = (j / nr) * 8 + xcd;
         rest = j % nr;
     } else {
         pair = idx % P;
         rest = idx / P;
     }
-    const int rep = rest % p.n_rep;
-    const int qt = p.n_qtiles - 1 - rest / p.n_rep;
+    const int rep = rest % p.n_rep, slot = rest / p.n_rep;
     const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
+    // A slot is one q tile (late, heavier tiles first) or, when the host paired them, a late tile and its early
+    // counterpart: under a causal mask every block then has the same amount of work.
+    const bool paired = p.n_slots != p.n_qtiles;
+#pragma nounroll
+    for (int part = 0; part < 2; part++) {
+    const int qt = part == 0 ? p.n_qtiles - 1 - slot : slot;
+    if (part == 1 && (!paired || qt >= p.n_qtiles - 1 - slot)) break;
+    if (part == 1) __syncthreads();   // the first tile's epilogue used the LDS buffers as staging areas
+    // the lane index is made opaque per tile: everything derived from it (LDS addresses of the tile loop ...) is then
+    // computed inside the tile's own scope instead of being hoisted out of this loop and kept alive across the epilogue
+    int lane_of_part = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane_of_part));
+    const int lane = lane_of_part, l32 = lane & 31, hh = lane >> 5;
 
     const int row0 = qt * BM;
     const int my_row = row0 + w * 32 + l32;
@@ -787,6 +801,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             it++;
         });
     }
+    }   // part
 }
 
 // ------------------------------------------------------------------------------ forward, fp32
@@ -1420,7 +1435,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     int idx = blockIdx.x, pair, rest;
     const int P = p.B * p.Hkv;
     if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3, nr = ((p.Sq + BM - 1) / BM) * p.n_rep;
+        int xcd = idx & 7, j = idx >> 3, nr = p.n_slots * p.n_rep;
         pair = (j / nr) * 8 + xcd;
         rest = j % nr;
     } else {
@@ -1428,9 +1443,18 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
         rest = idx / P;
     }
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int rep = rest % p.n_rep;
-    const int qt = n_qt - 1 - rest / p.n_rep;
+    const int rep = rest % p.n_rep, slot = rest / p.n_rep;
     const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
+    // one q tile per block (late tiles first) or a late tile and its early counterpart (see q_tile_slots)
+    const bool paired = p.n_slots != n_qt;
+#pragma nounroll
+    for (int part = 0; part < 2; part++) {
+    const int qt = part == 0 ? n_qt - 1 - slot : slot;
+    if (part == 1 && (!paired || qt >= n_qt - 1 - slot)) break;
+    if (part == 1) __syncthreads();   // the first tile's epilogue used the LDS buffers as staging areas
+    int lane_of_part = threadIdx.x & 63;   // opaque per tile, see the forward kernel
+    asm volatile("" : "+v"(lane_of_part));
+    const int lane = lane_of_part, l32 = lane & 31, hh = lane >> 5;
 
     const int row0 = qt * BM;
     const int my_row = row0 + w * 32 + l32;
@@ -1657,6 +1681,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
             });
         }
     }
+    }   // part
 }
 
 // ------------------------------------------------------------------------------ backward, fp32
@@ -1933,6 +1958,20 @@ bool strides_ok(const int64_t *s, int elem_bytes) {
 
 int fits_i32(int64_t x) { return x >= 0 && x < (int64_t)0x7fffffff; }
 
+// Slots of q tiles handed to the blocks of the forward and dQ kernels.  Under a causal mask a tile's work grows with its
+// rows' positions; pairing tile t with tile n - 1 - t in one block gives every block the same work (no long blocks left
+// over at the end of the launch) and halves the number of blocks to start.  Only done while the equal blocks still fill
+// the device's CUs evenly; otherwise one tile per slot, heaviest first, and the hardware's in-order dispatch balances.
+int q_tile_slots(int n_qtiles, long long blocks_per_tile, bool causal) {
+    if (!causal || n_qtiles < 2) return n_qtiles;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (cus <= 0) cus = 256;
+    const int n_slots = (n_qtiles + 1) / 2;
+    const long long n = n_slots * blocks_per_tile, rounds = (n + cus - 1) / cus;
+    return n * 10 >= rounds * cus * 9 ? n_slots : n_qtiles;
+}
+
 // every position of the local rows lies inside the rows [pos0, pos0 + len) of a RoPE table
 bool rope_table_covers(const int64_t *q_pos0, int64_t q_split, int64_t Sq, int64_t pos0, int64_t len) {
     if (len <= 0 || !fits_i32(pos0)) return false;
@@ -2055,14 +2094,16 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     if (a->io_dtype == LTR_BF16) {
         p.n_qtiles = (p.Sq + 255) / 256;
-        const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
-        if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+        if ((long long)p.n_qtiles * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
+        p.n_slots = q_tile_slots(p.n_qtiles, (long long)p.B * p.Hq, (p.flags & LTR_CAUSAL) != 0);
+        const long long nblk = (long long)p.n_slots * p.B * p.Hq;
         rc = enable_large_lds();
         if (rc) return rc;
         if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<128>(), st, p);
         else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<64>(), st, p);
     } else {
         p.n_qtiles = (p.Sq + 63) / 64;
+        p.n_slots = p.n_qtiles;
         const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
         if (nblk > 0x7fffffffLL) return LTR_EINVAL;
         if (a->D == 128) hipLaunchKernelGGL(fwd_f32_kernel<128>, dim3((unsigned)nblk), dim3(64), 0, st, p);
@@ -2220,8 +2261,9 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     }
     rc = enable_large_lds();
     if (rc) return rc;
-    const long long nblk_q = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
-    if (nblk_q > 0x7fffffffLL) return LTR_EINVAL;
+    if ((long long)((p.Sq + 255) / 256) * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
+    p.n_slots = q_tile_slots((p.Sq + 255) / 256, (long long)p.B * p.Hq, (flags & LTR_CAUSAL) != 0);
+    const long long nblk_q = (long long)p.n_slots * p.B * p.Hq;
     // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
     if (do_dq) {
         if (a->D == 128) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
