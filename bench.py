@@ -429,12 +429,55 @@ def _bench_mfma_ceiling(args):
     print(json.dumps(out), flush=True)
 
 
+def _bench_dq_atomics(args):
+    """The rate at which 64 x 128 fp32 partial dQ tiles can be added into memory with global atomics (ltr_probe_atomic_tile_add):
+    what a backward that produced dQ inside the key-owning blocks would need, beside what it needs at the dK/dV kernel's
+    speed."""
+    import torch
+    import lightron_amd as la
+    torch.cuda.set_device(0)
+    lib = la._lib.load()
+    n = 8192 + (1 << 20)
+    g = torch.Generator().manual_seed(1)
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    ws[8192:] = ((torch.rand((n - 8192) // 2, generator=g) * 4 - 2).to(torch.bfloat16)).view(torch.uint8).cuda()
+    dst = torch.zeros(32, 4096, 128, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    steps = 512
+    res = {}
+    for key, with_mfma in (("atomic_adds_only", 0), ("atomic_adds_between_40_mfma_per_wave", 1)):
+        best = None
+        for _ in range(3):
+            dst.zero_()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            la._lib.check(lib.ltr_probe_atomic_tile_add(dst.data_ptr(), dst.numel(), ws.data_ptr(), n, steps, with_mfma, stream),
+                          "ltr_probe_atomic_tile_add")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            best = ms if best is None or ms < best else best
+        ok = bool((dst == steps / 8).all().item())
+        res[key] = {"ms": round(best, 3), "us_per_tile_per_block": round(best * 1e3 / steps, 3),
+                    "payload_TB_per_s": round(256 * steps * 32768 / (best * 1e-3) / 1e12, 3), "sums_correct": ok}
+    # MFMA-only time of the same loop, for the share of the adds in the combined run: 40 MFMA per wave and step
+    need = {"step_us_at_dkdv_speed": 2.06, "payload_TB_per_s_needed": round(256 * 32768 / 2.06e-6 / 1e12, 2),
+            "note": "a 5-GEMM step of 64 rows x 128 keys x 4 slices per CU takes about 2.06 us at 1300 TFLOP/s; one 32 KiB tile add per step"}
+    out = {"metric": "fp32 global-atomic tile-add rate (partial dQ of a fused backward)", "value": res["atomic_adds_only"]["payload_TB_per_s"],
+           "unit": "TB/s", "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "256 blocks x 8 waves, each block adds one 64 x 128 fp32 tile per step into a [32, 4096, 128] buffer shared like dQ"},
+           "results": res, "needed_by_a_fused_backward": need}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling", "dq_atomics"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other workloads and the device probe")
     args = ap.parse_args()
@@ -448,6 +491,8 @@ def main():
         return _bench_rope(args)
     if args.workload == "mfma_ceiling":
         return _bench_mfma_ceiling(args)
+    if args.workload == "dq_atomics":
+        return _bench_dq_atomics(args)
     la._lib.load()
     torch.cuda.set_device(0)
     cfg = _workload(args.workload)

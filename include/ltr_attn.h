@@ -281,8 +281,19 @@ typedef struct ltr_device_info_t {
 
 #define LTR_PROBE_MIN_WORKSPACE (8192 + 65536)
 
+ /*
+ * ltr_probe_atomic_tile_add - the rate at which blocks can ADD 64 x 128 fp32 tiles into shared memory with global
+ * atomics: what a backward that produced dQ inside the key-owning blocks would have to sustain (one tile per block
+ * per 64-row step; at the attention kernels' speed that is one every ~2 us per CU, ~4 TB/s of fp32 payload over the
+ * device).  256 blocks of 8 waves; every block adds `steps` tiles (value 1.0 per element, coalesced: a half-wave = 128
+ * contiguous bytes of one row) into dst, fp32 [32][4096][128], zero-filled by the caller: afterwards every element
+ * holds steps / 8 (steps a multiple of 256).  with_mfma != 0: 40 MFMAs per wave between two adds, the matrix work of
+ * such a step.  workspace as for ltr_probe_mfma (operands from bytes [8192, ...)).  Timed by the caller with events.
+ */
 int ltr_device_info(ltr_device_info_t *out);
 int ltr_probe_mfma(void *workspace, int64_t workspace_bytes, int32_t iters, int32_t random_operands, void *stream);
+int ltr_probe_atomic_tile_add(float *dst, int64_t dst_elems, void *workspace, int64_t workspace_bytes, int32_t steps,
+                              int32_t with_mfma, void *stream);
 
 int ltr_abi_version(void);
 const char *ltr_strerror(int code);

@@ -16,7 +16,7 @@ LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LT
 LTR_ROPE_Q, LTR_ROPE_DQ = 128, 256
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
-           "ltr_device_info", "ltr_probe_mfma", "ltr_abi_version", "ltr_strerror")
+           "ltr_device_info", "ltr_probe_mfma", "ltr_probe_atomic_tile_add", "ltr_abi_version", "ltr_strerror")
 
 _i64x3 = ctypes.c_int64 * 3
 _i64x2 = ctypes.c_int64 * 2
@@ -108,6 +108,9 @@ def load():
     lib.ltr_device_info.restype = ctypes.c_int
     lib.ltr_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
     lib.ltr_probe_mfma.restype = ctypes.c_int
+    lib.ltr_probe_atomic_tile_add.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32,
+                                              ctypes.c_int32, ctypes.c_void_p]
+    lib.ltr_probe_atomic_tile_add.restype = ctypes.c_int
     lib.ltr_abi_version.argtypes = []
     lib.ltr_abi_version.restype = ctypes.c_int
     lib.ltr_strerror.argtypes = [ctypes.c_int]
