@@ -827,6 +827,42 @@ def test_fused_rope_prologue_and_dq_epilogue(ltr, D, Hq, Hkv, Sq, q_pos, chunks,
     assert _rel(acc.cpu(), dq_ref) < GRAD_RTOL_BF16
 
 
+@pytest.mark.parametrize("D,B,Hq,Hkv,Sq,q_pos,split,chunks", [
+    (128, 8, 32, 32, 700, (0, 0), None, [(0, 700)]),                       # 3 q tiles: a pair and the middle tile alone
+    (64, 8, 32, 8, 1100, (300, 300), None, [(0, 1000), (1000, 400)]),      # 5 q tiles, ragged, GQA, two chunks
+    (128, 4, 64, 16, 1024, (0, 3072), 512, [(0, 512), (512, 2560), (3072, 512)]),   # zig-zag rows: two segments
+])
+def test_paired_q_tiles_forward_backward(ltr, D, B, Hq, Hkv, Sq, q_pos, split, chunks):
+    """Enough (batch, head) pairs that the host hands the forward and dQ kernels a late q tile and its early counterpart
+    per block (q_tile_slots: causal, and the equal blocks fill the 256 CUs evenly).  Odd tile counts (the middle tile runs
+    alone), a ragged last tile, GQA, both head dims, two-segment rows; against the dense oracle."""
+    g = torch.Generator().manual_seed(77 + Sq)
+    n_qt = (Sq + 255) // 256
+    n_slots = (n_qt + 1) // 2
+    blocks = n_slots * B * Hq
+    assert blocks * 10 >= -(-blocks // 256) * 256 * 9, "shape does not trigger the pairing"
+    sp = Sq if split is None else split
+    qpos = torch.cat([torch.arange(sp) + q_pos[0], torch.arange(Sq - sp) + q_pos[1]])
+    q, do = _randn((B, Sq, Hq, D), g, torch.bfloat16), _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    ks = [_randn((B, n, Hkv, D), g, torch.bfloat16) for _, n in chunks]
+    vs = [_randn((B, n, Hkv, D), g, torch.bfloat16) for _, n in chunks]
+    kpos = torch.cat([torch.arange(n) + p0 for p0, n in chunks])
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), torch.cat(ks, 1).float(), torch.cat(vs, 1).float(),
+                                                                       do.float(), qpos, kpos, True, dtype=torch.float32)
+    qd = q.cuda().requires_grad_(True)
+    kd = [k.cuda().requires_grad_(True) for k in ks]
+    vd = [v.cuda().requires_grad_(True) for v in vs]
+    o, lse = ltr.block_attention(qd, kd, vd, [p0 for p0, _ in chunks], q_pos, split, True)
+    o.backward(do.cuda())
+    assert (o.detach().cpu().float() - o_ref).abs().max() < O_TOL_BF16
+    fin = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert (lse.cpu()[fin] - lse_ref[fin]).abs().max() < LSE_TOL_BF16
+    assert _rel(qd.grad.cpu(), dq_ref) < GRAD_RTOL_BF16
+    assert _rel(torch.cat([k.grad for k in kd], 1).cpu(), dk_ref) < GRAD_RTOL_BF16
+    assert _rel(torch.cat([v.grad for v in vd], 1).cpu(), dv_ref) < GRAD_RTOL_BF16
+
+
 @pytest.mark.parametrize("seed", list(range(8)))
 def test_rope_sweep_bit_exact(ltr, seed):
     """ltr_rope_apply on random shapes, dtypes, layouts and starting positions against the oracle, bit for bit."""
