@@ -94,6 +94,60 @@ def test_no_alloc_entry_point_validation_without_gpu():
     assert lib.ltr_attn_bwd_noalloc(ctypes.byref(a), None) == -2      # bf16 only
 
 
+def test_fused_rope_validation_without_gpu():
+    L, lib = _lib()
+    a = L.FwdArgs()
+    a.q = a.o = a.lse = 4096
+    a.B, a.Hq, a.Hkv, a.D, a.Sq, a.n_chunks, a.q_split = 1, 4, 2, 128, 64, 1, 64
+    a.io_dtype = a.o_dtype = L.LTR_BF16
+    a.flags = L.LTR_ROPE_Q
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -1            # no table
+    a.rope_freqs, a.rope_pos0, a.rope_len = 4096, 0, 32
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -1            # table ends before the last row's position
+    a.rope_len = 64
+    a.q_pos0[0] = a.q_pos0[1] = 10
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -1            # rows at positions 10 .. 73
+    a.rope_pos0 = 10
+    a.rope_freqs = 4100
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -3            # misaligned table
+    a.rope_freqs, a.io_dtype, a.o_dtype = 4096, L.LTR_F32, L.LTR_F32
+    assert lib.ltr_attn_fwd(ctypes.byref(a), None) == -2            # bf16 only
+    b = L.BwdArgs()
+    b.q = b.d_o = b.lse = b.delta = b.dq = 4096
+    b.B, b.Hq, b.Hkv, b.D, b.Sq, b.n_chunks, b.q_split = 1, 4, 2, 128, 64, 1, 64
+    b.io_dtype = L.LTR_BF16
+    b.flags = L.LTR_ROPE_DQ | L.LTR_NO_DQ
+    b.rope_freqs, b.rope_len = 4096, 64
+    assert lib.ltr_attn_bwd(ctypes.byref(b), None) == -1            # the rotation lives in the dQ kernel's epilogue
+
+
+def test_bench_traffic_figure_is_tied_to_the_kernel_source(tmp_path, monkeypatch):
+    """bench.py takes roofline.traffic from the counter profile only while the kernel source still has the hash the
+    profile names: a changed source must give None (a stale figure is never reported)."""
+    import hashlib
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_mod", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    src = tmp_path / "k.hip"
+    src.write_text("kernel text")
+    prof = tmp_path / "counters.md"
+    digest = hashlib.sha256(src.read_bytes()).hexdigest()
+    prof.write_text("x\nkernel-source-sha256: %s\ntraffic-bytes-per-launch bwd_dkdv_kernel<128>: 1.2988e+09\n" % digest)
+    monkeypatch.setattr(bench, "KERNEL_SOURCE", str(src))
+    monkeypatch.setattr(bench, "COUNTER_PROFILE", str(prof))
+    val, why = bench._measured_traffic("bwd_dkdv_kernel<128>")
+    assert val == 1.2988e9 and digest[:12] in why
+    assert bench._measured_traffic("fwd_bf16_kernel<128>")[0] is None      # no line for that kernel
+    src.write_text("kernel text, edited")
+    val, why = bench._measured_traffic("bwd_dkdv_kernel<128>")
+    assert val is None and "stale" in why
+    # the committed profile and the committed source: either in step (a number) or flagged, never an exception
+    monkeypatch.undo()
+    val, why = bench._measured_traffic("bwd_dkdv_kernel<128>")
+    assert (val is None) or val > 0
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     from lightron_amd import _lib as L
     monkeypatch.setattr(L, "_lib", None)
