@@ -52,6 +52,47 @@ def test_no_alloc_backward_two_calls(ltr):
     _case(ltr, 13, 1, 4, 1, 128, 96, [96], False)
 
 
+def test_forward_and_no_alloc_backward_replay_in_a_hip_graph(ltr):
+    """The library neither allocates nor synchronises nor records memset nodes, so one forward + backward (DELTA in the
+    library's scratch array) can be captured in a HIP graph once the per-device set-up has happened in an eager call.  The
+    graph is replayed on fresh inputs several times, with eager work and synchronisations between the replays, and every
+    replay must give the eager call's bits."""
+    B, Hq, Hkv, D, S = 2, 8, 2, 128, 384
+    g = torch.Generator().manual_seed(5)
+    mk = lambda h: torch.randn(B, S, h, D, generator=g).to(torch.bfloat16).cuda()
+    q, k, v, do = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    o = torch.empty_like(q)
+    lse = torch.empty(B, Hq, S, dtype=torch.float32, device="cuda")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)      # bf16 results written by the kernels
+
+    def step():
+        ltr.attn_fwd(q, [k], [v], [0], 0, None, True, out=o, lse=lse)
+        ltr.attn_bwd_accumulate(q, do, lse, None, [k], [v], [0], dq, [dk], [dv], 0, None, True, o=o, library_scratch=True)
+
+    step()                                   # eager: per-device set-up (LDS opt-in, scratch address) happens here
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    for it in range(3):
+        for t in (q, k, v, do):
+            t.copy_(torch.randn(t.shape, generator=g).to(torch.bfloat16))
+        for t in (o, dq, dk, dv):
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (o, lse, dq, dk, dv)]
+        assert all(torch.isfinite(t.float()).all() for t in got)
+        step()                               # eager, same inputs
+        torch.cuda.synchronize()
+        for a, b, name in zip(got, (o, lse, dq, dk, dv), ("O", "LSE", "dQ", "dK", "dV")):
+            assert torch.equal(a, b), "%s of replay %d differs from the eager call" % (name, it)
+
+
 def test_no_alloc_rejects_what_it_cannot_hold(ltr):
     from lightron_amd import _lib as L
     lib = L.load()
