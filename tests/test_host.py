@@ -148,6 +148,16 @@ def test_bench_traffic_figure_is_tied_to_the_kernel_source(tmp_path, monkeypatch
     assert (val is None) or val > 0
 
 
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0 and "ONE GPU" in (res.stderr + res.stdout)
+    env = dict(os.environ, WORLD_SIZE="2")
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")], capture_output=True, text=True, env=env)
+    assert res.returncode != 0 and "ONE GPU" in (res.stderr + res.stdout)
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     from lightron_amd import _lib as L
     monkeypatch.setattr(L, "_lib", None)
