@@ -535,6 +535,11 @@ def main():
         others["c4_rope"] = _run_c4_rope(la, torch, 5, 2)
         out["other_workloads"] = others
     out["device"] = _device_report(la, torch, probe=not args.no_others)
+    if "mfma_loop_random_operands" in out["device"]:
+        # beside the fraction of the published peak: the fraction of what a pure MFMA loop sustains on THIS box on random data
+        ceil = out["device"]["mfma_loop_random_operands"]["tflops"]
+        out["frac_of_measured_mfma_ceiling"] = round(tflops / ceil, 4)
+        out["roofline"]["frac_of_measured_mfma_ceiling"] = round(achieved / ceil, 4)
     if not args.no_cpu_baseline:
         # the host's cores as the box presents them; OMP_NUM_THREADS (set on the GPU boxes to the job's CPU share) caps
         # the threads actually used
