@@ -29,6 +29,11 @@
 //                        the same backward in scalar fp32 (no MFMA), for the 1e-4 parity cases.
 //   The tile loops of the bf16 kernels are unrolled over their LDS buffers (or, where registers are short,
 //   keep per-lane LDS addresses in registers): no address arithmetic is left between the MFMAs.
+//   RoPE: with LTR_ROPE_Q the forward rotates each q row in its operand registers (rope_rotate8) and can store the
+//   rotated row; with LTR_ROPE_DQ the dQ kernel's epilogue rotates dQ by the conjugate angles (rope_conj4).
+//   Block scheduling under a causal mask: a forward / dQ block takes a late q tile and its early counterpart when the
+//   host says so (q_tile_slots), and the dK/dV kernel's chunk table is sorted by position (longest blocks first).
+//   ltr_attn_bwd_noalloc keeps its DELTA workspace in the fixed __device__ array `scratch` (see there).
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, i = l % 32, h = l / 32):
 //   A[i][8h .. 8h+7], B[8h .. 8h+7][i], C[8*(r/4) + 4h + r%4][i] for accumulator register r.
