@@ -217,10 +217,11 @@ def _device_report(la, torch, probe=True):
     return rep
 
 
-def _run_attention(la, torch, cfg, steps, warmup):
+def _run_attention(la, torch, cfg, steps, warmup, data="randn"):
     """Times `steps` steps of one workload after `warmup` untimed ones; inputs are resident in HBM before the timed
     region.  Returns the step time, the credited flops and the average launch time of each kernel (HIP events on the
-    stream the kernels are launched on)."""
+    stream the kernels are launched on).  data="zeros" replaces the workload's N(0,1) inputs by zeros (same kernels, same
+    instruction stream, no toggling operand bits): only used by _data_dependence."""
     dev = torch.device("cuda:0")
     B, Hq, Hkv, D, S, W = (cfg[x] for x in ("B", "Hq", "Hkv", "D", "S", "W"))
     causal, bwd = cfg["causal"], cfg["bwd"]
@@ -230,6 +231,8 @@ def _run_attention(la, torch, cfg, steps, warmup):
     g = torch.Generator().manual_seed(0)
     def mk(h):
         full = torch.randn(B, S, h, D, generator=g).to(torch.bfloat16)
+        if data == "zeros":
+            full.zero_()
         return torch.stack([full[:, _rank_positions(cfg, r)] for r in range(W)], 0).to(dev)
     q_all, k_all, v_all = mk(Hq), mk(Hkv), mk(Hkv)
     do_all = mk(Hq) if bwd else None
@@ -337,6 +340,25 @@ def _run_attention(la, torch, cfg, steps, warmup):
         dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_share
     return {"dt": dt, "f_total": f_total, "kernels": kernels, "launches": launches,
             "dominant": (dom, dom_flops / (dom_ms * 1e-3) / 1e12)}
+
+
+def _data_dependence(la, torch, cfg):
+    """The same three kernels on one rank share of the workload, once on its N(0,1) inputs and once on all-zero inputs
+    (identical launches and instruction streams).  Executed TFLOP/s of each kernel: on zeros the chip keeps its full
+    clock, on random data the matrix pipe's switching activity runs it into the power limit - the gap between the
+    two is the clock, not the kernels' schedule."""
+    share = dict(cfg, ranks=cfg["ranks"][:1])
+    out = {"what": "executed TFLOP/s per kernel, one rank share, same launches on N(0,1) inputs and on all-zero inputs"}
+    for data in ("randn", "zeros", "randn", "zeros"):
+        r = _run_attention(la, torch, share, 6, 3, data=data)
+        k = r["kernels"]
+        cur = {"fwd_bf16_kernel": k["fwd_bf16_kernel"]["algorithmic_tflops"]}
+        if cfg["bwd"]:
+            cur["bwd_dkdv_kernel"] = k["bwd_dkdv_kernel"]["algorithmic_tflops"]
+            cur["bwd_dq_kernel"] = k["bwd_dq_kernel"]["executed_tflops"]
+        key = "n01_inputs" if data == "randn" else "zero_inputs"
+        out[key] = {n: max(v, out.get(key, {}).get(n, 0.0)) for n, v in cur.items()}
+    return out
 
 
 def _run_c4_rope(la, torch, steps, warmup):
@@ -534,6 +556,8 @@ def main():
         torch.cuda.empty_cache()
         others["c4_rope"] = _run_c4_rope(la, torch, 5, 2)
         out["other_workloads"] = others
+        torch.cuda.empty_cache()
+        out["data_dependence"] = _data_dependence(la, torch, cfg)
     out["device"] = _device_report(la, torch, probe=not args.no_others)
     if "mfma_loop_random_operands" in out["device"]:
         # beside the fraction of the published peak: the fraction of what a pure MFMA loop sustains on THIS box on random data
