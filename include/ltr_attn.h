@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 5
+#define LTR_ABI_VERSION 6
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -56,6 +56,9 @@ extern "C" {
 #define LTR_DKDV_BF16 64u /* backward: chunk[c].dk / dv are bf16 tensors that RECEIVE dK / dV of this call (no accumulation) */
 #define LTR_ROPE_Q 128u   /* forward: q is un-rotated; RoPE is applied to it in the kernel's prologue (rope_freqs) */
 #define LTR_ROPE_DQ 256u  /* backward: dQ leaves the dQ kernel rotated by the conjugate angles (gradient of LTR_ROPE_Q) */
+#define LTR_DKDV_KEYS_128 512u  /* backward, tuning hint: the dK/dV kernel's blocks own 128 keys (the default choice is the library's) */
+#define LTR_DKDV_KEYS_256 1024u /* backward, tuning hint: they own 256 keys (bf16, head dim 64 only: LTR_EUNSUP otherwise); results
+                                   do not depend on the hint beyond the order of fp32 additions inside a block */
 
 /* error codes */
 #define LTR_OK 0
@@ -184,7 +187,8 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;
-    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ |
+                             LTR_DKDV_KEYS_128 | LTR_DKDV_KEYS_256 */
     int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: scalar fp32 kernels for the 1e-4 parity cases;
                              LTR_DQ_BF16, LTR_DELTA_FROM_O and LTR_DKDV_BF16 are bf16 only and return LTR_EUNSUP with it) */
     int32_t n_chunks;

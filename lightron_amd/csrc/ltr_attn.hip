@@ -21,6 +21,11 @@
 //                        go global -> LDS directly into three swizzled buffers, one barrier
 //                        per tile; K, V operands and the dK^T / dV^T accumulators stay in
 //                        registers for the whole block.
+//   bwd_dkdv_wide_kernel<64>
+//                        the same kernel with two 32-key halves per wave (256 keys per block): every Q / dO operand
+//                        read from LDS feeds two MFMAs, and a block's transfers and per-step costs are spread over
+//                        twice the matrix work.  The registers allow it at head dim 64 only; chosen by the host
+//                        when the blocks are long and still many (or forced with LTR_DKDV_KEYS_256).
 //   bwd_dq_kernel<D>     forward-shaped: a block owns 256 query rows, loops over K/V tiles
 //                        (same direct-to-LDS tiles as the forward), recomputes S and dP and
 //                        accumulates dQ^T in registers.  No atomics anywhere: results are
@@ -1419,6 +1424,523 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     }
 }
 
+// lds_gemm_chain / lds_tr_gemm for a wave that owns KW 32-key halves: every operand read from LDS feeds one MFMA per half
+// (b[k], r[k] / acc[k] belong to half k); hook(step) follows the MFMAs of operand `step`.
+template <int D, int KW, class Hook = NoHook>
+__device__ __forceinline__ void lds_gemm_chain_kw(const __bf16 *row, int sw, const bf16x8 (&b)[KW][D / 16], f32x16 (&r)[KW],
+                                                  Hook hook = Hook()) {
+    constexpr int NK = D / 16, PF = 2;
+    bf16x8 x[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF; i++) x[i] = *(const bf16x8 *)(row + (((2 * i) ^ sw) << 3));
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + PF < NK) x[(kb + PF) % (PF + 1)] = *(const bf16x8 *)(row + (((2 * (kb + PF)) ^ sw) << 3));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < KW; k++) r[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[kb % (PF + 1)], b[k][kb], r[k], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        hook(kb);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+template <int D, int NKB, int KW, class Hook = NoHook>
+__device__ __forceinline__ void lds_tr_gemm_kw(const __bf16 *T, int row0, int lane, const bf16x8 (&b)[KW][NKB],
+                                               f32x16 (&acc)[KW][D / 32], Hook hook = Hook()) {
+    constexpr int ND = D / 32, N = NKB * ND, PF = 3;
+    bf16x8 a[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF && i < N; i++) a[i] = lds_operand_tr_swz<D>(T, row0 + (i / ND) * 16, (i % ND) * 32, lane);
+#pragma unroll
+    for (int step = 0; step < N; step++) {
+        if (step + PF < N)
+            a[(step + PF) % (PF + 1)] = lds_operand_tr_swz<D>(T, row0 + ((step + PF) / ND) * 16, ((step + PF) % ND) * 32, lane);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < KW; k++)
+            acc[k][step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[k][step / ND], acc[k][step % ND], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        hook(step);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// LDS of bwd_dkdv_wide_kernel: as BwdLds with 256 keys per block (64 per wave pair) and twice the P slots
+template <int D>
+struct BwdLdsWide {
+    static constexpr int BN = 256;
+    static constexpr int BM = 64;
+    static constexpr int NT = 512;
+    static constexpr int TILE = BM * D;
+    static constexpr int BUF_BYTES = 2 * TILE * 2 + 3 * BM * 4;
+    static constexpr int P_SLOT = 64 * 32;
+    static constexpr int NBUF = 3;
+    static constexpr int P_OFF = NBUF * BUF_BYTES;
+    static constexpr int MAX_QTILES = 4096;
+    static constexpr int LIST_OFF = P_OFF + 4 * 4 * 2 * P_SLOT;           // 4 slices x 2 parities x 2 sub-tiles x 2 halves
+    static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;
+    static_assert(TOTAL >= 8 * WaveStage<D>::BYTES, "the epilogue's staging areas reuse this memory");
+    static_assert(TOTAL <= 160 * 1024, "LDS of one CU");
+};
+
+// bwd_dkdv_kernel with two 32-key halves per wave (a block owns 256 keys): per MFMA half the LDS operand reads, half the
+// Q / dO transfers and half the per-step costs.  Fits the register file at head dim 64 only.
+template <int D>
+__global__ __launch_bounds__(512) void bwd_dkdv_wide_kernel(const BwdParams p) {
+    using L = BwdLdsWide<D>;
+    constexpr int KW = 2;   // 32-key halves per wave
+    constexpr int BN = L::BN, BM = L::BM;
+    constexpr int CPR = D / 8;
+    constexpr int RPI = 64 / CPR;        // rows filled by one wave-wide LDS-direct load (1 KB)
+    constexpr int NI = BM / (RPI * 8);   // such loads per wave, per tensor and per tile
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slice = w & 3;             // 64-key slice; waves w and w+4 (same SIMD) are partners
+    const bool p_role = w < 4;           // P wave (S, P, dV) or dS wave (dP, dS, dK)
+    const int l32 = lane & 31, hh = lane >> 5;
+    const bool causal = p.flags & LTR_CAUSAL;
+
+    // block -> (batch, kv head, chunk, key tile); same XCD grouping as the forward
+    int idx = blockIdx.x, pair, rest;
+    const int P = p.B * p.Hkv;
+    if ((P & 7) == 0) {
+        int xcd = idx & 7, j = idx >> 3;
+        pair = (j / p.tiles_total) * 8 + xcd;
+        rest = j % p.tiles_total;
+    } else {
+        pair = idx % P;
+        rest = idx / P;
+    }
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv;
+    int c = 0, kt = rest;
+    for (; c < p.n_chunks; c++) {
+        int n = (p.chunk[c].sk + BN - 1) / BN;
+        if (kt < n) break;
+        kt -= n;
+    }
+    if (c >= p.n_chunks) return;
+    const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
+    const int key0 = kt * BN;
+    int my_key[KW];   // this lane's keys in the S / dP / dK^T / dV^T tiles of the wave's two halves
+    bool key_ok[KW];
+#pragma unroll
+    for (int k = 0; k < KW; k++) {
+        my_key[k] = key0 + slice * 32 * KW + 32 * k + l32;
+        key_ok[k] = my_key[k] < sk;
+    }
+    const int tile_kpos_lo = pos0 + key0;
+    const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
+    const bool key_tail = key0 + BN > sk;
+    if (causal) {   // no query of this launch sees the block (a later chunk of the ring): nothing to add, nothing to load
+        int q_lo, q_hi;
+        q_pos_range(0, (int)p.Sq - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], q_lo, q_hi);
+        if (q_hi < tile_kpos_lo) {
+            for (int k = 0; k < KW; k++)
+            if ((p.flags & LTR_DKDV_BF16) && key_ok[k]) {   // results, not accumulators: these keys get zeros
+                __bf16 *gz = p_role ? (__bf16 *)p.chunk[c].dv + b * p.dvs[0] + (long long)my_key[k] * p.dvs[1] + hkv * p.dvs[2]
+                                    : (__bf16 *)p.chunk[c].dk + b * p.dks[0] + (long long)my_key[k] * p.dks[1] + hkv * p.dks[2];
+                for (int d = 8 * hh; d < D; d += 16) *(uint4 *)(gz + d) = make_uint4(0, 0, 0, 0);
+            }
+            return;
+        }
+    }
+
+    // resident B operand: K rows for a P wave, V rows for a dS wave; lane (key l32, half hh) holds
+    // d = 16*kb + 8*hh .. +7
+    bf16x8 kvreg[KW][D / 16];
+    {
+        const __bf16 *base = p_role ? (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2]
+                                    : (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+        const long long rs = p_role ? p.ks[1] : p.vs[1];
+#pragma unroll
+        for (int k = 0; k < KW; k++) {
+            const int ksafe = min(my_key[k], sk - 1);
+#pragma unroll
+            for (int kb = 0; kb < D / 16; kb++) {
+                uint4 x = *(const uint4 *)(base + (long long)ksafe * rs + kb * 16 + 8 * hh);
+                if (!key_ok[k]) x = make_uint4(0, 0, 0, 0);
+                kvreg[k][kb] = as_bf16x8(x);
+            }
+        }
+    }
+
+    f32x16 zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+    f32x16 acc[KW][D / 32];              // dV^T (P wave) or dK^T (dS wave) of the two halves
+#pragma unroll
+    for (int k = 0; k < KW; k++)
+#pragma unroll
+        for (int i = 0; i < D / 32; i++) acc[k][i] = zero16;
+    const float c2 = p.scale * LTR_LOG2E;
+
+    // A tile's class depends on its rows only: 0 = no row sees any key of the block (skipped);
+    // 1 = every (row, key) pair is visible; 2 = needs the mask (diagonal, tails).
+    auto tile_class = [&](int qt) {
+        const int row0 = qt * BM;
+        const bool edge = key_tail || row0 + BM > p.Sq;
+        if (!causal) return edge ? 2 : 1;
+        int lo, hi;
+        q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
+        if (hi < tile_kpos_lo) return 0;
+        return (edge || tile_kpos_hi > lo) ? 2 : 1;
+    };
+
+    // The q tiles of each class are listed once per block (wave 0, ballot compaction: the order, and with it
+    // the rounding of the accumulation, is fixed), so the main loops carry no classification arithmetic.
+    unsigned short *const tlist = (unsigned short *)(smem + L::LIST_OFF);     // [2][MAX_QTILES]
+    int *const tcount = (int *)(smem + L::LIST_OFF + 2 * L::MAX_QTILES * 2);
+    if (w == 0) {
+        int n1 = 0, n2 = 0;
+        for (int base = 0; base < p.n_qtiles; base += 64) {
+            const int qt = base + lane;
+            const int cls = qt < p.n_qtiles ? tile_class(qt) : 0;
+            const unsigned long long m1 = __builtin_amdgcn_ballot_w64(cls == 1), m2 = __builtin_amdgcn_ballot_w64(cls == 2);
+            const unsigned long long below = (1ull << lane) - 1ull;
+            if (cls == 1) tlist[n1 + __builtin_popcountll(m1 & below)] = (unsigned short)qt;
+            if (cls == 2) tlist[L::MAX_QTILES + n2 + __builtin_popcountll(m2 & below)] = (unsigned short)qt;
+            n1 += __builtin_popcountll(m1);
+            n2 += __builtin_popcountll(m2);
+        }
+        if (lane == 0) {
+            tcount[0] = n1;
+            tcount[1] = n2;
+        }
+    }
+    __syncthreads();
+
+    const int st_row = lane / CPR, st_pc = lane % CPR;   // this lane's place inside a 1 KB LDS-direct load
+    const float st_mul = tid < BM ? -1.f / p.scale : -1.f;  // threads 0..63 stage -LSE/scale, 64..127 stage -DELTA
+    float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
+    bool sld_ok = true;
+    int sld_row0 = 0;     // first row of the tile in flight
+    unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * KW * (L::P_SLOT / 4);   // [parity][sub-tile][half]
+
+    // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
+    // live in straight-line loop bodies and the unmasked pass carries no bounds checks at all
+    auto run_pass = [&](auto mask_tag) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr int cls = MASK ? 2 : 1;
+        const int cnt = __builtin_amdgcn_readfirstlane(tcount[cls - 1]);
+        const unsigned short *const list = tlist + (cls - 1) * L::MAX_QTILES;
+        int li_ = -1;                                 // index into the list
+        // the list entry of the next call is read from LDS one call ahead, so its latency is never waited for
+        unsigned short pre = list[0];
+        auto advance = [&](int &rep, int &qt) {   // next tile of this class after (rep, qt); false when done
+            if (++li_ >= cnt) {
+                li_ = 0;
+                if (++rep >= p.n_rep) return false;
+            }
+            qt = __builtin_amdgcn_readfirstlane((int)pre);
+            pre = list[li_ + 1 < cnt ? li_ + 1 : 0];
+            return true;
+        };
+        // Q and dO tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane): wave w
+        // fills rows RPI*(NI*w + i) .. of both tiles with its i-th pair of loads, lane l the chunk position
+        // l % CPR of row l / CPR, fetching the logical chunk the swizzle places there.  Rows past the end of Q
+        // repeat its last row (they are masked).  LSE and DELTA go through a register of threads 0..127.
+        auto gload = [&](int rep, int qt, int buf) {
+            const int h = hkv * p.n_rep + rep;
+            const int row0 = qt * BM;
+            sld_row0 = row0;
+            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
+            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
+            const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
+            const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
+            const unsigned Qd = lds_address(smem) + buf * L::BUF_BYTES, dOd = Qd + L::TILE * 2;   // LDS byte addresses
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                const int row = RPI * (NI * w + i) + st_row;
+                const int grow = MASK ? min(row0 + row, p.Sq - 1) : row0 + row;
+                const int chunk = st_pc ^ lds_swz<D>(row);
+                global_to_lds_b128(qp + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D * 2);
+                global_to_lds_b128(dop + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D * 2);
+            }
+            if (tid < 2 * BM) {
+                if (!MASK) {
+                    sld = sp[tid];
+                } else {
+                    const int r = tid < BM ? tid : tid - BM;
+                    sld_ok = row0 + r < p.Sq;
+                    sld = sp[sld_ok ? tid : (tid < BM ? 0 : BM)];
+                }
+            }
+        };
+        auto lds_store = [&](int buf) {   // the LSE / DELTA values fetched by gload
+            float *st = (float *)(smem + buf * L::BUF_BYTES) + L::TILE;   // after the two bf16 tiles
+            if (tid < 2 * BM) {
+                float x = sld * st_mul;
+                // rows past the end: -LSE/scale = -inf makes P = 0 (they are masked as well)
+                if (MASK) x = sld_ok ? x : (tid < BM ? -INFINITY : 0.f);
+                st[tid] = x;
+            } else if (MASK && tid < 3 * BM) {   // positions of the tile's rows (third wave)
+                const int row = sld_row0 + tid - 2 * BM;
+                ((int *)st)[tid] = row >= p.Sq ? BWD_QPOS_NONE
+                                   : causal ? q_position(row, p.q_split, p.q_pos0[0], p.q_pos0[1]) : BWD_QPOS_ALL;
+            }
+        };
+
+        int kpos[KW];
+#pragma unroll
+        for (int k = 0; k < KW; k++) kpos[k] = key_ok[k] ? pos0 + my_key[k] : BWD_KPOS_NONE;
+        if (cnt == 0) return;
+        int rep = 0, qt = 0;
+        advance(rep, qt);
+        __syncthreads();   // the previous pass has finished reading LDS
+        gload(rep, qt, 0);
+        lds_store(0);
+        tile_barrier();
+        // One LDS barrier per 64-row tile.  In step t the P wave does all its work on tile t (S of both
+        // sub-tiles, P -> slots of parity t & 1, dV) and the dS wave all its work on tile t-1 (dP, dS with P
+        // from the slots filled one step earlier, dK): inside a step the two waves of a SIMD are independent,
+        // so one wave's softmax arithmetic runs under the other's MFMAs.  Slots of parity (t & 1) are
+        // rewritten in step t+2, after the barrier that ends step t+1 in which they were read.  Tile t+1 is
+        // fetched into registers at the start of step t and stored at its end into buffer (t+1) % 3, which
+        // held tile t-2, last read in step t-1.  Both roles execute T + 1 barriers.
+        auto put_slot = [&](unsigned *slot, const PackedTile &t) {
+            // two 16-byte halves per lane, each half contiguous over the lanes (no bank conflicts)
+            *(uint4 *)(slot + lane * 4) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
+            *(uint4 *)(slot + 256 + lane * 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
+        };
+        int par = 0;
+        // In the pass over unmasked tiles both loops are unrolled over the three Q / dO buffers (buf is a compile-time
+        // constant inside a step), so that LDS addresses are loop-invariant per-lane registers plus immediate offsets;
+        // the pass over masked tiles (few steps, more live registers) keeps one loop body with buf in a register.
+        if (p_role) {
+            bool more = true;
+            auto p_step = [&](auto buf_tag) {
+                const int buf = buf_tag;
+                more = advance(rep, qt);
+                const int nbuf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                if (more) gload(rep, qt, nbuf);
+                const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
+                const __bf16 *dOs = Qs + L::TILE;
+                const float *st_s = (const float *)(dOs + L::TILE);   // -LSE/scale of the tile's rows
+                unsigned *slots = pslot_base + par * 2 * KW * (L::P_SLOT / 4);
+                // Accumulator register r of a sub-tile <-> tile row 8*(r/4) + 4*hh + r%4: both S accumulators start at
+                // -LSE/scale of their rows.  Order of the step: S of sub-tile a; S of sub-tile b with the
+                // exponentials of a issued under its MFMAs; first half of dV (rows of a) with the exponentials of b
+                // under its MFMAs; second half of dV.
+                f32x16 sa[KW], sb[KW];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 la = *(const f32x4 *)(st_s + 8 * g + 4 * hh), lb = *(const f32x4 *)(st_s + 32 + 8 * g + 4 * hh);
+#pragma unroll
+                    for (int k = 0; k < KW; k++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            sa[k][4 * g + e] = la[e];
+                            sb[k][4 * g + e] = lb[e];
+                        }
+                }
+                int qa[16], qb[16];   // positions of the rows (masked tiles only)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int *st_q = (const int *)st_s + 2 * BM;
+                    const i32x4 xa = MASK ? *(const i32x4 *)(st_q + 8 * g + 4 * hh) : i32x4{0, 0, 0, 0};
+                    const i32x4 xb = MASK ? *(const i32x4 *)(st_q + 32 + 8 * g + 4 * hh) : i32x4{0, 0, 0, 0};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        qa[4 * g + e] = xa[e];
+                        qb[4 * g + e] = xb[e];
+                    }
+                }
+                PackedTile ppa[KW], ppb[KW];
+                constexpr int NK = D / 16, ND = D / 32;
+                __builtin_amdgcn_s_setprio(1);
+                // every Q / dO operand read from LDS feeds the MFMAs of both halves
+                lds_gemm_chain_kw<D, KW>(Qs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, sa);
+                lds_gemm_chain_kw<D, KW>(Qs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, sb, [&](int kb) {
+#pragma unroll
+                    for (int k = 0; k < KW; k++)
+#pragma unroll
+                        for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) ppa[k].u[j] = bwd_p_pair<MASK>(sa[k], j, c2, kpos[k], qa);
+                });
+                bf16x8 pba[KW][2], pbb[KW][2];
+#pragma unroll
+                for (int k = 0; k < KW; k++) {
+                    put_slot(slots + k * (L::P_SLOT / 4), ppa[k]);
+                    pba[k][0] = operand_of(ppa[k], 0);
+                    pba[k][1] = operand_of(ppa[k], 1);
+                }
+                lds_tr_gemm_kw<D, 2, KW>(dOs, 0, lane, pba, acc, [&](int step) {
+#pragma unroll
+                    for (int k = 0; k < KW; k++)
+#pragma unroll
+                        for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) ppb[k].u[j] = bwd_p_pair<MASK>(sb[k], j, c2, kpos[k], qb);
+                });
+#pragma unroll
+                for (int k = 0; k < KW; k++) {
+                    put_slot(slots + (KW + k) * (L::P_SLOT / 4), ppb[k]);
+                    pbb[k][0] = operand_of(ppb[k], 0);
+                    pbb[k][1] = operand_of(ppb[k], 1);
+                }
+                lds_tr_gemm_kw<D, 2, KW>(dOs, 32, lane, pbb, acc);
+                __builtin_amdgcn_s_setprio(0);
+                if (more) lds_store(nbuf);
+                tile_barrier();
+                par ^= 1;
+            };
+            static_assert(L::NBUF == 3, "unrolled over three buffers");
+            if (MASK) {
+                int buf = 0;
+                while (more) {
+                    p_step(buf);
+                    buf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                }
+            } else {
+                for (;;) {
+                    p_step(std::integral_constant<int, 0>{});
+                    if (!more) break;
+                    p_step(std::integral_constant<int, 1>{});
+                    if (!more) break;
+                    p_step(std::integral_constant<int, 2>{});
+                    if (!more) break;
+                }
+            }
+            tile_barrier();                        // step T: only the dS waves have work
+        } else {
+            bool more = advance(rep, qt);          // step 0: staging duties only
+            if (more) gload(rep, qt, 1);
+            tile_barrier();
+            bool had_next = true;
+            auto ds_step = [&](auto buf_tag) {
+                const int buf = buf_tag;
+                had_next = more;
+                if (more) {
+                    more = advance(rep, qt);
+                    if (more) gload(rep, qt, buf + 2 >= L::NBUF ? buf + 2 - L::NBUF : buf + 2);
+                }
+                const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
+                const __bf16 *dOs = Qs + L::TILE;
+                const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
+                const unsigned *slots = pslot_base + par * 2 * KW * (L::P_SLOT / 4);
+                // the dP accumulators start at -DELTA of their rows (register r <-> tile row 8*(r/4) + 4*hh + r%4);
+                // same order as the P wave: dP of a; dP of b with dS of a under its MFMAs; first half of dK with dS of
+                // b under its MFMAs; second half of dK
+                f32x16 dpa[KW], dpb[KW];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 da = *(const f32x4 *)(dlt_s + 8 * g + 4 * hh), db4 = *(const f32x4 *)(dlt_s + 32 + 8 * g + 4 * hh);
+#pragma unroll
+                    for (int k = 0; k < KW; k++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            dpa[k][4 * g + e] = da[e];
+                            dpb[k][4 * g + e] = db4[e];
+                        }
+                }
+                PackedTile dsa[KW], dsb[KW];
+                constexpr int NK = D / 16, ND = D / 32;
+                __builtin_amdgcn_s_setprio(1);
+                lds_gemm_chain_kw<D, KW>(dOs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, dpa);
+                unsigned pua[KW][8], pub[KW][8];
+#pragma unroll
+                for (int k = 0; k < KW; k++) {
+                    const unsigned *sl = slots + k * (L::P_SLOT / 4);
+                    const uint4 pa0 = *(const uint4 *)(sl + lane * 4), pa1 = *(const uint4 *)(sl + 256 + lane * 4);
+                    pua[k][0] = pa0.x; pua[k][1] = pa0.y; pua[k][2] = pa0.z; pua[k][3] = pa0.w;
+                    pua[k][4] = pa1.x; pua[k][5] = pa1.y; pua[k][6] = pa1.z; pua[k][7] = pa1.w;
+                }
+                lds_gemm_chain_kw<D, KW>(dOs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, dpb, [&](int kb) {
+#pragma unroll
+                    for (int k = 0; k < KW; k++)
+#pragma unroll
+                        for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) dsa[k].u[j] = bwd_ds_pair(pua[k][j], dpa[k], j);
+                });
+                bf16x8 dba[KW][2], dbb[KW][2];
+#pragma unroll
+                for (int k = 0; k < KW; k++) {
+                    const unsigned *sl = slots + (KW + k) * (L::P_SLOT / 4);
+                    const uint4 pb0 = *(const uint4 *)(sl + lane * 4), pb1 = *(const uint4 *)(sl + 256 + lane * 4);
+                    pub[k][0] = pb0.x; pub[k][1] = pb0.y; pub[k][2] = pb0.z; pub[k][3] = pb0.w;
+                    pub[k][4] = pb1.x; pub[k][5] = pb1.y; pub[k][6] = pb1.z; pub[k][7] = pb1.w;
+                    dba[k][0] = operand_of(dsa[k], 0);
+                    dba[k][1] = operand_of(dsa[k], 1);
+                }
+                lds_tr_gemm_kw<D, 2, KW>(Qs, 0, lane, dba, acc, [&](int step) {
+#pragma unroll
+                    for (int k = 0; k < KW; k++)
+#pragma unroll
+                        for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) dsb[k].u[j] = bwd_ds_pair(pub[k][j], dpb[k], j);
+                });
+#pragma unroll
+                for (int k = 0; k < KW; k++) {
+                    dbb[k][0] = operand_of(dsb[k], 0);
+                    dbb[k][1] = operand_of(dsb[k], 1);
+                }
+                lds_tr_gemm_kw<D, 2, KW>(Qs, 32, lane, dbb, acc);
+                __builtin_amdgcn_s_setprio(0);
+                tile_barrier();
+                par ^= 1;
+            };
+            if (MASK) {
+                int buf = 0;
+                while (had_next) {
+                    ds_step(buf);
+                    buf = buf == L::NBUF - 1 ? 0 : buf + 1;
+                }
+            } else {
+                for (;;) {
+                    ds_step(std::integral_constant<int, 0>{});
+                    if (!had_next) break;
+                    ds_step(std::integral_constant<int, 1>{});
+                    if (!had_next) break;
+                    ds_step(std::integral_constant<int, 2>{});
+                    if (!had_next) break;
+                }
+            }
+        }
+    };
+    run_pass(std::false_type{});
+    run_pass(std::true_type{});
+
+    // dV^T (P wave) / dK^T (dS wave) tile of the wave's 32 keys: added to the fp32 accumulators in whole rows, through the
+    // wave's LDS staging area (every wave is past the last barrier: tiles, slots and lists are no longer read)
+#pragma unroll
+    for (int k = 0; k < KW; k++) {
+        constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
+        const long long stride = uniform64(p_role ? p.dvs[1] : p.dks[1]);
+        const int key_base = uniform32(key0 + slice * 32 * KW + 32 * k), sk_u = uniform32(sk);
+        const long long goff = (p_role ? b * p.dvs[0] + hkv * p.dvs[2] : b * p.dks[0] + hkv * p.dks[2]) +
+                               (key_base + lane / LPR) * stride + 4 * (lane % LPR);
+        if (uniform32(p.flags & LTR_DKDV_BF16)) {   // every query that sees these keys was in this launch: store the result
+            __bf16 *gb = (__bf16 *)(p_role ? p.chunk[c].dv : p.chunk[c].dk) + goff;
+            wave_tile_rowmajor<D>(smem + w * WaveStage<D>::BYTES, lane, acc[k], p_role ? 1.f : p.scale, [&](int row, int, f32x4 val) {
+                if (key_base + row < sk_u) {
+                    bf16x4 y;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
+                    *(bf16x4 *)gb = y;
+                }
+                gb += ROWS_PER_IT * stride;
+            });
+            continue;
+        }
+        float *gp = (p_role ? p.chunk[c].dv : p.chunk[c].dk) + goff;
+        // all reads of the accumulator first (independent loads in flight together), then the adds and the writes
+        constexpr int NIT = 32 / ROWS_PER_IT;
+        f32x4 old[NIT];
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (key_base + it * ROWS_PER_IT + lane / LPR < sk_u) old[it] = *(const f32x4 *)(gp + it * ROWS_PER_IT * stride);
+        }
+        int it = 0;
+        wave_tile_rowmajor<D>(smem + w * WaveStage<D>::BYTES, lane, acc[k], p_role ? 1.f : p.scale, [&](int row, int, f32x4 val) {
+            if (key_base + row < sk_u) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) val[e] += old[it][e];
+                *(f32x4 *)gp = val;
+            }
+            gp += ROWS_PER_IT * stride;
+            it++;
+        });
+    }
+}
+
 // dQ: same block / wave / lane roles as the forward (a lane owns one query row), so LSE and DELTA are
 // per-lane scalars.  S^T = K Q^T and dP^T = V dO^T with K, V tiles natural in LDS; dS^T leaves the
 // registers as the B operand of dQ^T += K^T dS^T, whose A operand is the K tile read by transpose loads.
@@ -1938,6 +2460,8 @@ int enable_large_lds() {
                                   BwdLds<128>::TOTAL) == hipSuccess &&
               hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   BwdLds<64>::TOTAL) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dkdv_wide_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  BwdLdsWide<64>::TOTAL) == hipSuccess &&
               hipFuncSetAttribute((const void *)fwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   fwd_lds_bytes<128>()) == hipSuccess &&
               hipFuncSetAttribute((const void *)fwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -2158,7 +2682,10 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     if (do_dq && !a->dq) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ)) return LTR_EINVAL;
+    if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ | LTR_DKDV_KEYS_128 |
+                  LTR_DKDV_KEYS_256))
+        return LTR_EINVAL;
+    if ((flags & LTR_DKDV_KEYS_128) && (flags & LTR_DKDV_KEYS_256)) return LTR_EINVAL;
     const bool fused_delta = flags & LTR_DELTA_FROM_O;
     if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
@@ -2190,6 +2717,23 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         p.rope = a->rope_freqs;
         p.rope_pos0 = (int)a->rope_pos0;
     }
+    // keys per block of the dK/dV kernel: 256 (two 32-key halves per wave) pays at head dim 64 when a block walks many q tiles
+    // and the wider blocks still fill the device several times over; the caller can force either size
+    bool wide = false;
+    if (flags & LTR_DKDV_KEYS_256) {
+        if (a->D != 64 || f32) return LTR_EUNSUP;
+        wide = true;
+    } else if (!(flags & LTR_DKDV_KEYS_128) && a->D == 64 && !f32 && do_dkdv) {
+        long long blocks256 = 0;
+        for (int c = 0; c < a->n_chunks; c++) blocks256 += (a->chunk[c].sk + 255) / 256;
+        blocks256 *= (long long)a->B * a->Hkv;
+        const long long steps = (long long)(a->Hq / a->Hkv) * ((a->Sq + 63) / 64) / ((flags & LTR_CAUSAL) ? 2 : 1);
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (cus <= 0) cus = 256;
+        wide = steps >= 48 && blocks256 >= (long long)((flags & LTR_CAUSAL) ? 4 : 2) * cus;
+    }
+    const int keys_per_block = wide ? BwdLdsWide<64>::BN : 128;
     long long tiles = 0;
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];
@@ -2204,7 +2748,7 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         p.chunk[c].dv = (float *)ch.dv;
         p.chunk[c].sk = (int)ch.sk;
         p.chunk[c].pos0 = (int)ch.pos0;
-        tiles += (ch.sk + 127) / 128;
+        tiles += (ch.sk + keys_per_block - 1) / keys_per_block;
     }
     int rc = check_device();
     if (rc) return rc;
@@ -2282,6 +2826,7 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         if (flags & LTR_CAUSAL)
             std::stable_sort(p.chunk, p.chunk + p.n_chunks, [](const ChunkDev &x, const ChunkDev &y) { return x.pos0 < y.pos0; });
         if (a->D == 128) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
+        else if (wide) hipLaunchKernelGGL(bwd_dkdv_wide_kernel<64>, dim3((unsigned)nblk), dim3(BwdLdsWide<64>::NT), BwdLdsWide<64>::TOTAL, st, p);
         else hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;

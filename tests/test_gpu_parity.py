@@ -879,3 +879,78 @@ def test_rope_sweep_bit_exact(ltr, seed):
     ref, _ = orc.apply_rotary_emb(xv, xv, fc)
     got, _ = ltr.apply_rotary_emb(xv.cuda(), xv.cuda(), fc.cuda())
     assert got.dtype == dtype and torch.equal(got.cpu(), ref)
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_dkdv_block_size_hints_d64(ltr, seed):
+    """Head dim 64: the dK/dV kernel with 128 and with 256 keys per block (LTR_DKDV_KEYS_128 / _256, the latter two 32-key
+    halves per wave), forced through the hint flags on shapes that the library's own choice would not send to the wide
+    kernel: ragged chunks that end inside a 256-key block, several chunks, GQA, causal with a two-segment query, fp32
+    accumulators and bf16 results.  Both against the dense oracle, and against each other to rounding."""
+    import random
+    rnd = random.Random(7000 + seed)
+    g = torch.Generator().manual_seed(8000 + seed)
+    D = 64
+    Hkv = rnd.choice([1, 2])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    B = rnd.choice([1, 2])
+    Sq = rnd.choice([64, 100, 256, 300, 513, 700])
+    n_ch = rnd.randint(1, 3)
+    sks = [rnd.choice([1, 33, 100, 128, 191, 256, 257, 330, 512, 600]) for _ in range(n_ch)]
+    causal = rnd.random() < 0.6
+    direct = rnd.random() < 0.5          # bf16 results instead of fp32 accumulators
+    starts, p = [], rnd.randint(0, 30)
+    for sk in sks:
+        starts.append(p)
+        p += sk + rnd.randint(0, 20)
+    q_split = rnd.choice([None, rnd.randint(1, Sq - 1)])
+    if q_split is None:
+        qp = rnd.randint(0, p)
+        q_pos, q_pos0 = torch.arange(qp, qp + Sq), qp
+    else:
+        a0, a1 = rnd.randint(0, p), rnd.randint(0, p + 100)
+        q_pos = torch.cat([torch.arange(a0, a0 + q_split), torch.arange(a1, a1 + Sq - q_split)])
+        q_pos0 = (a0, a1)
+    q = _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    do = _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    kbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
+    vbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
+    offs = [sum(sks[:i]) for i in range(n_ch)]
+    k_pos = torch.cat([torch.arange(starts[i], starts[i] + sks[i]) for i in range(n_ch)])
+    _, _, _, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), kbuf.float(), vbuf.float(), do.float(), q_pos, k_pos, causal)
+    qd, dod, kd, vd = _dev(q, do, kbuf, vbuf)
+    ks = [kd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    vs = [vd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    o, lse = ltr.attn_fwd(qd, ks, vs, starts, q_pos0, q_split, causal)
+    delta = ltr.attn_delta(o, dod)
+    got = {}
+    for keys in (128, 256):
+        dt = torch.bfloat16 if direct else torch.float32
+        dkb = torch.full(kbuf.shape, 7.0 if direct else 0.0, dtype=dt, device="cuda")   # results overwrite, accumulators add
+        dvb = torch.full(vbuf.shape, 7.0 if direct else 0.0, dtype=dt, device="cuda")
+        dks = [dkb[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+        dvs = [dvb[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+        dq = torch.zeros(q.shape, dtype=torch.float32, device="cuda")
+        ltr.attn_bwd_accumulate(qd, dod, lse, delta, ks, vs, starts, dq, dks, dvs, q_pos0, q_split, causal, do_dq=False,
+                                dkdv_keys=keys)
+        got[keys] = (dkb.float().cpu(), dvb.float().cpu())
+        for x, ref in ((got[keys][0], dk_ref), (got[keys][1], dv_ref)):
+            if ref.abs().max() > 0:
+                assert _rel(x, ref) < GRAD_RTOL_BF16, (keys, seed)
+            else:
+                assert x.abs().max() < 1e-3
+    for a, b_ in zip(got[128], got[256]):
+        assert (a - b_).abs().max() <= 2e-2 * max(1.0, b_.abs().max().item())
+
+
+def test_dkdv_keys_256_refused_where_it_does_not_exist(ltr):
+    g = torch.Generator().manual_seed(1)
+    q, k, v, do = (_randn((1, 64, 2, 128), g, torch.bfloat16).cuda() for _ in range(4))
+    o, lse = ltr.attn_fwd(q, [k], [v], [0])
+    delta = ltr.attn_delta(o, do)
+    dq = torch.zeros(q.shape, dtype=torch.float32, device="cuda")
+    dk, dv = torch.zeros_like(dq), torch.zeros_like(dq)
+    with pytest.raises(RuntimeError):
+        ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dkdv_keys=256)
+    with pytest.raises(RuntimeError):
+        ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dkdv_keys=64)
