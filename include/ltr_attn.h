@@ -59,6 +59,8 @@ extern "C" {
 #define LTR_DKDV_KEYS_128 512u  /* backward, tuning hint: the dK/dV kernel's blocks own 128 keys (the default choice is the library's) */
 #define LTR_DKDV_KEYS_256 1024u /* backward, tuning hint: they own 256 keys (bf16, head dim 64 only: LTR_EUNSUP otherwise); results
                                    do not depend on the hint beyond the order of fp32 additions inside a block */
+#define LTR_DQ_ROWS_256 2048u /* backward, tuning hint: the dQ kernel's blocks own 256 query rows (the default choice is the library's) */
+#define LTR_DQ_ROWS_512 4096u /* backward, tuning hint: they own 512 rows (bf16, head dim 64 only: LTR_EUNSUP otherwise); same results */
 
 /* error codes */
 #define LTR_OK 0
@@ -188,7 +190,7 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_split;
     float scale;
     uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ |
-                             LTR_DKDV_KEYS_128 | LTR_DKDV_KEYS_256 */
+                             LTR_DKDV_KEYS_128 | LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_256 | LTR_DQ_ROWS_512 */
     int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: scalar fp32 kernels for the 1e-4 parity cases;
                              LTR_DQ_BF16, LTR_DELTA_FROM_O and LTR_DKDV_BF16 are bf16 only and return LTR_EUNSUP with it) */
     int32_t n_chunks;

@@ -15,6 +15,7 @@ LTR_BF16, LTR_F32 = 0, 1
 LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LTR_DKDV_BF16 = 1, 2, 4, 8, 16, 32, 64
 LTR_ROPE_Q, LTR_ROPE_DQ = 128, 256
 LTR_DKDV_KEYS_128, LTR_DKDV_KEYS_256 = 512, 1024
+LTR_DQ_ROWS_256, LTR_DQ_ROWS_512 = 2048, 4096
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_device_info", "ltr_probe_mfma", "ltr_probe_atomic_tile_add", "ltr_abi_version", "ltr_strerror")

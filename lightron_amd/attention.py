@@ -152,7 +152,7 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
                         causal=False, scale=None, do_dq=True, do_dkdv=True, o=None, library_scratch=False, dq_rope=None,
-                        dkdv_keys=None):
+                        dkdv_keys=None, dq_rows=None):
     """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
     do_dq / do_dkdv select which of the two backward kernels are enqueued.  dq_acc may instead be a bf16
     tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
@@ -166,7 +166,8 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     required and the library allocates nothing.
     dq_rope: the (cos, sin) table of attn_fwd's q_rope; q is then the ROTATED q (q_rot_out of that forward) and the dQ
     kernel's epilogue rotates dQ back by the conjugate angles (LTR_ROPE_DQ): dq is the gradient of the un-rotated q.
-    dkdv_keys: None (the library chooses), 128 or 256 keys per block of the dK/dV kernel (256: bf16 with head dim 64 only)."""
+    dkdv_keys: None (the library chooses), 128 or 256 keys per block of the dK/dV kernel (256: bf16 with head dim 64 only).
+    dq_rows: None, 256 or 512 query rows per block of the dQ kernel (512: bf16 with head dim 64 only)."""
     lib = _lib.load()
     if library_scratch and (o is None or not do_dq):
         raise RuntimeError("library_scratch needs o (DELTA is computed from it) and do_dq")
@@ -209,6 +210,10 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
         if dkdv_keys not in (128, 256):
             raise RuntimeError("dkdv_keys must be None, 128 or 256")
         a.flags |= _lib.LTR_DKDV_KEYS_128 if dkdv_keys == 128 else _lib.LTR_DKDV_KEYS_256
+    if dq_rows is not None:
+        if dq_rows not in (256, 512):
+            raise RuntimeError("dq_rows must be None, 256 or 512")
+        a.flags |= _lib.LTR_DQ_ROWS_256 if dq_rows == 256 else _lib.LTR_DQ_ROWS_512
     if dq_rope is not None:
         _rope_table_check(dq_rope, D, q.device)
         if not do_dq:

@@ -26,6 +26,10 @@
 //                        read from LDS feeds two MFMAs, and a block's transfers and per-step costs are spread over
 //                        twice the matrix work.  The registers allow it at head dim 64 only; chosen by the host
 //                        when the blocks are long and still many (or forced with LTR_DKDV_KEYS_256).
+//   bwd_dq_wide_kernel<64>
+//                        bwd_dq_kernel with two 32-row blocks per wave (512 query rows per block, a lane owns two rows):
+//                        every K / V operand read from LDS feeds two MFMAs; head dim 64 only, chosen by the host when
+//                        the wider blocks still fill the device (or forced with LTR_DQ_ROWS_512).
 //   bwd_dq_kernel<D>     forward-shaped: a block owns 256 query rows, loops over K/V tiles
 //                        (same direct-to-LDS tiles as the forward), recomputes S and dP and
 //                        accumulates dQ^T in registers.  No atomics anywhere: results are
@@ -2211,6 +2215,352 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     }   // part
 }
 
+// lds_gemm_pair_at / lds_tr_gemm_at for a wave that owns RB 32-row blocks: every operand read from LDS feeds one MFMA per row
+// block (ba[rb], bb[rb], ra[rb], rb_[rb] / b[rb], acc[rb] belong to row block rb).
+template <int D, int RB>
+__device__ __forceinline__ void lds_gemm_pair_at_rb(const unsigned (&addr)[D / 16], int imm_a, int imm_b, const bf16x8 (&ba)[RB][D / 16],
+                                                    const bf16x8 (&bb)[RB][D / 16], f32x16 (&ra)[RB], f32x16 (&rb_)[RB]) {
+    constexpr int NK = D / 16, PF = 2;
+    bf16x8 xa[PF + 1], xb[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        xa[i] = *(lds_bf16x8_ptr)(uintptr_t)(addr[i] + imm_a);
+        xb[i] = *(lds_bf16x8_ptr)(uintptr_t)(addr[i] + imm_b);
+    }
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + PF < NK) {
+            xa[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(uintptr_t)(addr[kb + PF] + imm_a);
+            xb[(kb + PF) % (PF + 1)] = *(lds_bf16x8_ptr)(uintptr_t)(addr[kb + PF] + imm_b);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            ra[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[kb % (PF + 1)], ba[r][kb], ra[r], 0, 0, 0);
+            rb_[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xb[kb % (PF + 1)], bb[r][kb], rb_[r], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+template <int D, int NKB, int RB>
+__device__ __forceinline__ void lds_tr_gemm_at_rb(const unsigned (&addr)[D / 32][2], int imm, const bf16x8 (&b)[RB][NKB],
+                                                  f32x16 (&acc)[RB][D / 32]) {
+    constexpr int ND = D / 32, N = NKB * ND, PF = 3;
+    auto operand = [&](int i) {
+        const int off = imm + (i / ND) * 16 * D * 2;
+        union {
+            struct { i16x4 a, b; } s;
+            bf16x8 v;
+        } u;
+        u.s.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(addr[i % ND][0] + off));
+        u.s.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(addr[i % ND][1] + off));
+        return u.v;
+    };
+    bf16x8 a[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF && i < N; i++) a[i] = operand(i);
+#pragma unroll
+    for (int step = 0; step < N; step++) {
+        if (step + PF < N) a[(step + PF) % (PF + 1)] = operand(step + PF);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+            acc[r][step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[r][step / ND], acc[r][step % ND], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// bwd_dq_kernel with two 32-row blocks per wave (a block owns 512 query rows, a lane two of them): per MFMA half the LDS
+// operand reads, half the K / V transfers and half the per-tile costs.  Fits the register file at head dim 64 only.
+template <int D>
+__global__ __launch_bounds__(512) void bwd_dq_wide_kernel(const BwdParams p) {
+    constexpr int RB = 2;   // 32-row blocks per wave: a lane owns RB query rows
+    constexpr int NW = 8, BM = 32 * RB * NW, BN = FwdTile<D>::BN;   // 8 waves (two per SIMD) share every K / V tile
+    constexpr int CPR = D / 8;
+    constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
+    constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers,
+    constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
+    constexpr int BUF_ELEMS = 2 * TILE;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hh = lane >> 5;
+    const bool causal = p.flags & LTR_CAUSAL;
+
+    int idx = blockIdx.x, pair, rest;
+    const int P = p.B * p.Hkv;
+    if ((P & 7) == 0) {
+        int xcd = idx & 7, j = idx >> 3, nr = p.n_slots * p.n_rep;
+        pair = (j / nr) * 8 + xcd;
+        rest = j % nr;
+    } else {
+        pair = idx % P;
+        rest = idx / P;
+    }
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    const int rep = rest % p.n_rep, slot = rest / p.n_rep;
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
+    // one q tile per block (late tiles first) or a late tile and its early counterpart (see q_tile_slots)
+    const bool paired = p.n_slots != n_qt;
+#pragma nounroll
+    for (int part = 0; part < 2; part++) {
+    const int qt = part == 0 ? n_qt - 1 - slot : slot;
+    if (part == 1 && (!paired || qt >= n_qt - 1 - slot)) break;
+    if (part == 1) __syncthreads();   // the first tile's epilogue used the LDS buffers as staging areas
+    int lane_of_part = threadIdx.x & 63;   // opaque per tile, see the forward kernel
+    asm volatile("" : "+v"(lane_of_part));
+    const int lane = lane_of_part, l32 = lane & 31, hh = lane >> 5;
+
+    const int row0 = qt * BM;
+    int my_row[RB], my_pos[RB];
+    bool row_ok[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        my_row[rb] = row0 + w * 32 * RB + 32 * rb + l32;
+        row_ok[rb] = my_row[rb] < p.Sq;
+        my_pos[rb] = q_position(my_row[rb], p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    }
+    int blk_lo, blk_hi, w_lo, w_hi;
+    q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+    {
+        int wr0 = row0 + w * 32 * RB, wr1 = min(wr0 + 32 * RB, p.Sq) - 1;
+        if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
+        else { w_lo = -0x7fffffff; w_hi = -0x7fffffff; }  // wave has no valid row: everything masked
+    }
+
+    bf16x8 qreg[RB][D / 16], doreg[RB][D / 16];
+    float lse2[RB], dlt[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        lse2[rb] = INFINITY;
+        dlt[rb] = 0.f;
+        const int rsafe = min(my_row[rb], p.Sq - 1);
+        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + (long long)rsafe * p.qs[1] + h * p.qs[2];
+        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + (long long)rsafe * p.dos[1] + h * p.dos[2];
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) {
+            qreg[rb][kb] = as_bf16x8(*(const uint4 *)(qp + kb * 16 + 8 * hh));
+            doreg[rb][kb] = as_bf16x8(*(const uint4 *)(dop + kb * 16 + 8 * hh));
+        }
+        if (p.flags & LTR_DELTA_FROM_O) {
+            // DELTA = rowsum(dO * O) of this lane's row: its half of every 16-element block, then the other half's
+            const __bf16 *op = (const __bf16 *)p.o + b * p.os_[0] + (long long)rsafe * p.os_[1] + h * p.os_[2];
+            float part = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < D / 16; kb++) {
+                const bf16x8 ov = as_bf16x8(*(const uint4 *)(op + kb * 16 + 8 * hh));
+#pragma unroll
+                for (int e = 0; e < 8; e++) part += (float)ov[e] * (float)doreg[rb][kb][e];
+            }
+            dlt[rb] = xhalf_sum(part);
+            if (row_ok[rb] && hh == 0) p.delta[((long long)b * p.Hq + h) * p.Sq + my_row[rb]] = dlt[rb];
+        }
+        if (row_ok[rb]) {
+            // a row that saw no key has LSE = -inf: give it +inf like a row past the end, so that P = exp2(-inf) = 0
+            // whatever S is (S = -inf after the mask fix-up would otherwise meet -(-inf))
+            const float lse_row = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row[rb]];
+            lse2[rb] = lse_row == -INFINITY ? INFINITY : lse_row * LTR_LOG2E;
+            if (!(p.flags & LTR_DELTA_FROM_O)) dlt[rb] = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row[rb]];
+        }
+    }
+    f32x16 zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+    f32x16 dqacc[RB][D / 32];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int i = 0; i < D / 32; i++) dqacc[rb][i] = zero16;
+    const float c2 = p.scale * LTR_LOG2E;
+
+    // The fields of the chunk being loaded live in scalar registers and are re-read from the argument
+    // table only when the chunk changes (a scalar load per tile would share the LDS wait counter).
+    int c = -1, t = 0, nt = 0;
+    int ld_sk = 0, ld_pos0 = 0;
+    const __bf16 *ld_kb = nullptr, *ld_vb = nullptr;
+    auto settle = [&]() {
+        while (c < p.n_chunks && t >= nt) {
+            c++;
+            t = 0;
+            if (c < p.n_chunks) {
+                ld_sk = p.chunk[c].sk;
+                ld_pos0 = p.chunk[c].pos0;
+                ld_kb = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+                ld_vb = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+                const int nvis = causal ? max(0, min(ld_sk, blk_hi - ld_pos0 + 1)) : ld_sk;
+                nt = (nvis + BN - 1) / BN;
+            }
+        }
+    };
+    settle();
+
+    // Tiles go from global memory straight into LDS (see the forward kernel): wave w fills rows
+    // RPI*(NI*w + i) .. with its i-th load; rows past the end of a chunk repeat its last row and are masked.
+    const int st_row = lane / CPR, st_pc = lane % CPR;
+    int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
+    auto gload = [&](int ti, int buf) {
+        nx_sk = ld_sk;
+        nx_pos0 = ld_pos0;
+        nx_key0 = ti * BN;
+        const unsigned Kd = lds_address(smem) + buf * BUF_ELEMS * 2, Vd = Kd + TILE * 2;   // LDS byte addresses
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const int row = RPI * (NI * w + i) + st_row;
+            const int key = min(ti * BN + row, ld_sk - 1);
+            const int chunk = st_pc ^ lds_swz<D>(row);
+            global_to_lds_b128(ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8), Kd + RPI * (NI * w + i) * D * 2);
+            global_to_lds_b128(ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8), Vd + RPI * (NI * w + i) * D * 2);
+        }
+    };
+
+    bool have = c < p.n_chunks;
+    if (have) gload(t, 0);
+    tile_barrier();
+    // LDS byte addresses of this lane's operands in the K tile of the current buffer (the V tile and the other 32-key
+    // blocks are immediates away): kept in registers and flipped to the other buffer with one XOR each per tile
+    static_assert((BUF_ELEMS * 2 & (BUF_ELEMS * 2 - 1)) == 0, "buffer size must be a power of two for the XOR flip");
+    unsigned pa[D / 16], ta[D / 32][2];
+    {
+        const unsigned lds0 = lds_address(smem);   // the only LDS object of the kernel: aligned far beyond the buffer size
+        const int sw = lds_swz<D>(l32) ^ hh;        // rows l32 + 32 n share the swizzle word of row l32
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) pa[kb] = lds0 + ((l32 * D + (((2 * kb) ^ sw) << 3)) << 1);
+        const int li = lane & 15, g = lane >> 4;
+#pragma unroll
+        for (int j = 0; j < D / 32; j++)
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int col = j * 32 + ((g & 1) << 4) + ((li & 3) << 2), row = 4 * (g >> 1) + (li >> 2) + 8 * e;
+                ta[j][e] = lds0 + ((lds_swz_off<D>(row, col >> 3) + (col & 7)) << 1);
+            }
+    }
+    int par = 0;
+    while (have) {
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
+        t++;
+        settle();
+        const bool have_next = c < p.n_chunks;
+        if (have_next) gload(t, par ^ 1);
+
+        const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
+        // 32 keys at a time, one block after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
+        // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic.  A wave whose rows all
+        // precede the tile's first key has nothing to add (see the forward kernel).
+        if (!causal || pos0 + key0 <= w_hi) {
+#pragma unroll
+        for (int nb = 0; nb < BN / 32; nb++) {
+            f32x16 s[RB], dp[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                s[rb] = zero16;
+                dp[rb] = zero16;
+            }
+            __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
+            lds_gemm_pair_at_rb<D, RB>(pa, nb * 32 * D * 2, TILE * 2 + nb * 32 * D * 2, qreg, doreg, s, dp);
+            __builtin_amdgcn_s_setprio(0);
+            // mask fix-up (tail of the chunk, diagonal tiles, rows past the end): wave-uniform branch touching S only;
+            // an invisible entry gets S = -inf, so P = 0 and dS = 0
+            if (need_mask) {
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                        const bool vis = key < sk && row_ok[rb] && (!causal || pos0 + key <= my_pos[rb]);
+                        s[rb][r] = vis ? s[rb][r] : -INFINITY;
+                    }
+            }
+            bf16x8 dsb[RB][2];
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                PackedTile ds;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    float dsv[2];
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const int r = 2 * j + e;
+                        const float pv = __builtin_amdgcn_exp2f(s[rb][r] * c2 - lse2[rb]);
+                        dsv[e] = pv * (dp[rb][r] - dlt[rb]);
+                    }
+                    ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
+                }
+                dsb[rb][0] = operand_of(ds, 0);
+                dsb[rb][1] = operand_of(ds, 1);
+            }
+            __builtin_amdgcn_s_setprio(1);
+            lds_tr_gemm_at_rb<D, 2, RB>(ta, nb * 32 * D * 2, dsb, dqacc);   // every K^T operand feeds one MFMA per row block
+            __builtin_amdgcn_s_setprio(0);
+        }
+        }
+        tile_barrier();
+#pragma unroll
+        for (int kb = 0; kb < D / 16; kb++) pa[kb] ^= BUF_ELEMS * 2;
+#pragma unroll
+        for (int j = 0; j < D / 32; j++) {
+            ta[j][0] ^= BUF_ELEMS * 2;
+            ta[j][1] ^= BUF_ELEMS * 2;
+        }
+        par ^= 1;
+        have = have_next;
+    }
+
+    // dQ in whole rows through the wave's LDS staging area (the tiles are no longer read: the last barrier is behind us)
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
+        unsigned char *stage = smem + w * WaveStage<D>::BYTES;
+        const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + w * 32 * RB + 32 * rb);
+        const long long dqs1 = uniform64(p.dqs[1]);
+        const long long off0 = uniform64(b * p.dqs[0] + h * p.dqs[2]) + (wave_row0 + lane / LPR) * dqs1 + 4 * (lane % LPR);
+        // LTR_ROPE_DQ: q was rotated by the forward's prologue, so the gradient of the caller's un-rotated q is dQ rotated by
+        // the conjugate angles of its row's position (the rotation is linear: it commutes with the accumulation over calls)
+        const bool rope = uniform32(p.flags & LTR_ROPE_DQ) != 0;
+        const float *const rope_tab = p.rope;
+        const int rope_p0 = uniform32(p.rope_pos0), split_u = uniform32(p.q_split), qp0 = uniform32(p.q_pos0[0]), qp1 = uniform32(p.q_pos0[1]);
+        auto unrotate = [&](int row, int col, f32x4 val) {
+            if (!rope) return val;
+            const int pos = q_position(wave_row0 + row, split_u, qp0, qp1);
+            return rope_conj4(val, *(const f32x4 *)(rope_tab + (long long)(pos - rope_p0) * D + col));
+        };
+        if (uniform32(p.flags & LTR_DQ_BF16)) {   // this call saw every key of these rows: store the result, no accumulator
+            __bf16 *dqp = (__bf16 *)p.dq + off0;
+            wave_tile_rowmajor<D>(stage, lane, dqacc[rb], p.scale, [&](int row, int col, f32x4 val) {
+                if (wave_row0 + row < Sq_u) {
+                    val = unrotate(row, col, val);
+                    bf16x4 y;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
+                    *(bf16x4 *)dqp = y;
+                }
+                dqp += ROWS_PER_IT * dqs1;
+            });
+        } else {
+            float *dqp = (float *)p.dq + off0;
+            constexpr int NIT = 32 / ROWS_PER_IT;
+            f32x4 old[NIT];   // all reads of the accumulator first, then the adds and the writes
+#pragma unroll
+            for (int it = 0; it < NIT; it++) {
+                old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (wave_row0 + it * ROWS_PER_IT + lane / LPR < Sq_u) old[it] = *(const f32x4 *)(dqp + it * ROWS_PER_IT * dqs1);
+            }
+            int it = 0;
+            wave_tile_rowmajor<D>(stage, lane, dqacc[rb], p.scale, [&](int row, int col, f32x4 val) {
+                if (wave_row0 + row < Sq_u) {
+                    val = unrotate(row, col, val);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) val[e] += old[it][e];
+                    *(f32x4 *)dqp = val;
+                }
+                dqp += ROWS_PER_IT * dqs1;
+                it++;
+            });
+        }
+    }
+    }   // part
+}
+
 // ------------------------------------------------------------------------------ backward, fp32
 // The fp32 path (1e-4 parity cases, not a performance path): scalar FMAs like fwd_f32_kernel, no atomics.
 //   bwd_dq_f32_kernel    one query row per lane (q, dO, dQ in registers), K/V tiles of 32 keys broadcast from LDS
@@ -2469,6 +2819,8 @@ int enable_large_lds() {
               hipFuncSetAttribute((const void *)bwd_dq_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<128>()) == hipSuccess &&
               hipFuncSetAttribute((const void *)bwd_dq_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  dq_lds_bytes<64>()) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_wide_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<64>()) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
@@ -2683,15 +3035,17 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
     if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ | LTR_DKDV_KEYS_128 |
-                  LTR_DKDV_KEYS_256))
+                  LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_256 | LTR_DQ_ROWS_512))
         return LTR_EINVAL;
     if ((flags & LTR_DKDV_KEYS_128) && (flags & LTR_DKDV_KEYS_256)) return LTR_EINVAL;
+    if ((flags & LTR_DQ_ROWS_256) && (flags & LTR_DQ_ROWS_512)) return LTR_EINVAL;
     const bool fused_delta = flags & LTR_DELTA_FROM_O;
     if (fused_delta && (!do_dq || !a->o)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     const bool f32 = a->io_dtype == LTR_F32;
-    if (f32 && (flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ))) return LTR_EUNSUP;   // bf16 conveniences only
+    if (f32 && (flags & (LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ | LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_512)))
+        return LTR_EUNSUP;   // bf16 conveniences and kernels only
     const int gb = (flags & LTR_DKDV_BF16) ? 2 : 4;   // bytes per dK / dV element
     const int eb = f32 ? 4 : 2;
     if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
@@ -2811,11 +3165,29 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     rc = enable_large_lds();
     if (rc) return rc;
     if ((long long)((p.Sq + 255) / 256) * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
-    p.n_slots = q_tile_slots((p.Sq + 255) / 256, (long long)p.B * p.Hq, (flags & LTR_CAUSAL) != 0);
+    // query rows per block of the dQ kernel: 512 (two 32-row blocks per wave) pays at head dim 64 when the wider blocks still
+    // fill the device, and under a causal mask only on sequences long enough that the diagonal does not dominate
+    bool wide_q = false;
+    if (flags & LTR_DQ_ROWS_512) {
+        if (a->D != 64) return LTR_EUNSUP;
+        wide_q = true;
+    } else if (!(flags & LTR_DQ_ROWS_256) && a->D == 64 && do_dq) {
+        const bool causal_ = (flags & LTR_CAUSAL) != 0;
+        const int tiles512 = (p.Sq + 511) / 512, slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_);
+        const long long blocks512 = (long long)slots512 * p.B * p.Hq;
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (cus <= 0) cus = 256;
+        // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance
+        wide_q = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus) : (blocks512 * 4 >= (long long)cus * 3);
+    }
+    const int dq_rows = wide_q ? 512 : 256;
+    p.n_slots = q_tile_slots((p.Sq + dq_rows - 1) / dq_rows, (long long)p.B * p.Hq, (flags & LTR_CAUSAL) != 0);
     const long long nblk_q = (long long)p.n_slots * p.B * p.Hq;
     // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
     if (do_dq) {
         if (a->D == 128) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
+        else if (wide_q) hipLaunchKernelGGL(bwd_dq_wide_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
         else hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
     }
     if (do_dkdv) {

@@ -917,7 +917,7 @@ def test_dkdv_block_size_hints_d64(ltr, seed):
     vbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
     offs = [sum(sks[:i]) for i in range(n_ch)]
     k_pos = torch.cat([torch.arange(starts[i], starts[i] + sks[i]) for i in range(n_ch)])
-    _, _, _, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), kbuf.float(), vbuf.float(), do.float(), q_pos, k_pos, causal)
+    _, _, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(q.float(), kbuf.float(), vbuf.float(), do.float(), q_pos, k_pos, causal)
     qd, dod, kd, vd = _dev(q, do, kbuf, vbuf)
     ks = [kd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
     vs = [vd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
@@ -941,6 +941,23 @@ def test_dkdv_block_size_hints_d64(ltr, seed):
                 assert x.abs().max() < 1e-3
     for a, b_ in zip(got[128], got[256]):
         assert (a - b_).abs().max() <= 2e-2 * max(1.0, b_.abs().max().item())
+    # the dQ kernel with 256 and with 512 query rows per block (LTR_DQ_ROWS_256 / _512: two 32-row blocks per wave), fp32
+    # accumulator or bf16 result, DELTA given or computed from O by the kernel
+    gq = {}
+    for rows in (256, 512):
+        dq = (torch.full(q.shape, 7.0, dtype=torch.bfloat16, device="cuda") if direct
+              else torch.zeros(q.shape, dtype=torch.float32, device="cuda"))
+        dlt = torch.full_like(delta, float("nan")) if direct else delta
+        ltr.attn_bwd_accumulate(qd, dod, lse, dlt, ks, vs, starts, dq, ks, vs, q_pos0, q_split, causal, do_dkdv=False,
+                                o=o if direct else None, dq_rows=rows)
+        gq[rows] = dq.float().cpu()
+        if direct:
+            assert torch.allclose(dlt, delta, rtol=1e-5, atol=1e-5)
+        if dq_ref.abs().max() > 0:
+            assert _rel(gq[rows], dq_ref) < GRAD_RTOL_BF16, (rows, seed)
+        else:
+            assert gq[rows].abs().max() < 1e-3
+    assert (gq[256] - gq[512]).abs().max() <= 2e-2 * max(1.0, gq[512].abs().max().item())
 
 
 def test_dkdv_keys_256_refused_where_it_does_not_exist(ltr):
@@ -954,3 +971,5 @@ def test_dkdv_keys_256_refused_where_it_does_not_exist(ltr):
         ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dkdv_keys=256)
     with pytest.raises(RuntimeError):
         ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dkdv_keys=64)
+    with pytest.raises(RuntimeError):
+        ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dq_rows=512)
