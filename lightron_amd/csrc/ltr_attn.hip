@@ -13,7 +13,7 @@
 //                        with an earlier partial result is part of the epilogue.
 //   fwd_f32_kernel<D>    fp32 I/O and arithmetic (no MFMA), for the 1e-4 parity case.
 //   delta_kernel         DELTA = rowsum(dO * O).
-//   bwd_dkdv_kernel<D>   a block of 8 waves owns 128 keys of one kv head and loops over the
+//   bwd_dkdv_kernel<D, KW>  a block of 8 waves owns 128 * KW keys of one kv head and loops over the
 //                        query heads of the GQA group and over 64-row query tiles taken from
 //                        lists (fully visible / partly masked) built once in LDS.  Two waves
 //                        share each 32-key slice: one computes S, P and dV^T, the other dP,
@@ -21,19 +21,16 @@
 //                        go global -> LDS directly into three swizzled buffers, one barrier
 //                        per tile; K, V operands and the dK^T / dV^T accumulators stay in
 //                        registers for the whole block.
-//   bwd_dkdv_wide_kernel<64>
-//                        the same kernel with two 32-key halves per wave (256 keys per block): every Q / dO operand
+//                        bwd_dkdv_kernel<64, 2>: two 32-key halves per wave (256 keys per block): every Q / dO operand
 //                        read from LDS feeds two MFMAs, and a block's transfers and per-step costs are spread over
 //                        twice the matrix work.  The registers allow it at head dim 64 only; chosen by the host
 //                        when the blocks are long and still many (or forced with LTR_DKDV_KEYS_256).
-//   bwd_dq_wide_kernel<64>
-//                        bwd_dq_kernel with two 32-row blocks per wave (512 query rows per block, a lane owns two rows):
-//                        every K / V operand read from LDS feeds two MFMAs; head dim 64 only, chosen by the host when
-//                        the wider blocks still fill the device (or forced with LTR_DQ_ROWS_512).
-//   bwd_dq_kernel<D>     forward-shaped: a block owns 256 query rows, loops over K/V tiles
+//   bwd_dq_kernel<D, RB> forward-shaped: a block owns 256 * RB query rows, loops over K/V tiles
 //                        (same direct-to-LDS tiles as the forward), recomputes S and dP and
 //                        accumulates dQ^T in registers.  No atomics anywhere: results are
-//                        bitwise reproducible.
+//                        bitwise reproducible.  bwd_dq_kernel<64, 2>: two 32-row blocks per wave (a lane owns two
+//                        query rows): every K / V operand read from LDS feeds two MFMAs; head dim 64 only, chosen by the
+//                        host when the wider blocks still fill the device (or forced with LTR_DQ_ROWS_512).
 //   bwd_dq_f32_kernel<D>, bwd_dkdv_f32_kernel<D, DV>
 //                        the same backward in scalar fp32 (no MFMA), for the 1e-4 parity cases.
 //   The tile loops of the bf16 kernels are unrolled over their LDS buffers (or, where registers are short,
@@ -976,9 +973,9 @@ __global__ __launch_bounds__(256) void cast_kernel(const float *src, __bf16 *dst
 //                    dQ^T accumulates in registers.
 // LDS of bwd_dkdv_kernel (dynamic): three buffers of {Q tile, dO tile, -LSE/scale, -DELTA, row positions}, the P slots,
 // the tile lists.
-template <int D>
+template <int D, int KW>
 struct BwdLds {
-    static constexpr int BN = 128;      // keys per block, 32 per wave pair
+    static constexpr int BN = 128 * KW; // keys per block, 32 * KW per wave pair
     static constexpr int BM = 64;       // query rows per tile (two 32-row MFMA sub-tiles)
     static constexpr int NT = 512;      // threads per block
     static constexpr int TILE = BM * D;                                  // elements; rows unpadded, chunks swizzled
@@ -987,9 +984,10 @@ struct BwdLds {
     static constexpr int NBUF = 3;                                       // tile t (P waves), t-1 (dS waves), t+1 (in flight)
     static constexpr int P_OFF = NBUF * BUF_BYTES;
     static constexpr int MAX_QTILES = 4096;                              // Sq <= 262144 per launch
-    static constexpr int LIST_OFF = P_OFF + 4 * 4 * P_SLOT;              // 4 slices x 2 parities x 2 sub-tiles of P slots
+    static constexpr int LIST_OFF = P_OFF + 4 * 4 * KW * P_SLOT;         // 4 slices x 2 parities x 2 sub-tiles x KW halves of P slots
     static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;     // two tile lists (ushort) + counts
     static_assert(TOTAL >= 8 * WaveStage<D>::BYTES, "the epilogue's staging areas reuse this memory");
+    static_assert(TOTAL <= 160 * 1024, "LDS of one CU");
 };
 
 // Masked tiles: the visibility of (row, key) is kpos <= qpos[row], with the rows' positions staged in LDS beside LSE and
@@ -1015,417 +1013,6 @@ __device__ __forceinline__ unsigned bwd_p_pair(const f32x16 &sm, int j, float c2
 __device__ __forceinline__ unsigned bwd_ds_pair(unsigned pu, const f32x16 &dpm, int j) {
     const float p0 = __uint_as_float(pu << 16), p1 = __uint_as_float(pu & 0xffff0000u);
     return pack2_bf16(p0 * dpm[2 * j], p1 * dpm[2 * j + 1]);
-}
-
-template <int D>
-__global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
-    using L = BwdLds<D>;
-    constexpr int BN = L::BN, BM = L::BM;
-    constexpr int CPR = D / 8;
-    constexpr int RPI = 64 / CPR;        // rows filled by one wave-wide LDS-direct load (1 KB)
-    constexpr int NI = BM / (RPI * 8);   // such loads per wave, per tensor and per tile
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int slice = w & 3;             // 32-key slice; waves w and w+4 (same SIMD) are partners
-    const bool p_role = w < 4;           // P wave (S, P, dV) or dS wave (dP, dS, dK)
-    const int l32 = lane & 31, hh = lane >> 5;
-    const bool causal = p.flags & LTR_CAUSAL;
-
-    // block -> (batch, kv head, chunk, key tile); same XCD grouping as the forward
-    int idx = blockIdx.x, pair, rest;
-    const int P = p.B * p.Hkv;
-    if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3;
-        pair = (j / p.tiles_total) * 8 + xcd;
-        rest = j % p.tiles_total;
-    } else {
-        pair = idx % P;
-        rest = idx / P;
-    }
-    const int b = pair / p.Hkv, hkv = pair % p.Hkv;
-    int c = 0, kt = rest;
-    for (; c < p.n_chunks; c++) {
-        int n = (p.chunk[c].sk + BN - 1) / BN;
-        if (kt < n) break;
-        kt -= n;
-    }
-    if (c >= p.n_chunks) return;
-    const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
-    const int key0 = kt * BN;
-    const int my_key = key0 + slice * 32 + l32;   // this lane's key in S / dP / dK^T / dV^T tiles
-    const bool key_ok = my_key < sk;
-    const int tile_kpos_lo = pos0 + key0;
-    const int tile_kpos_hi = pos0 + min(key0 + BN, sk) - 1;
-    const bool key_tail = key0 + BN > sk;
-    if (causal) {   // no query of this launch sees the block (a later chunk of the ring): nothing to add, nothing to load
-        int q_lo, q_hi;
-        q_pos_range(0, (int)p.Sq - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], q_lo, q_hi);
-        if (q_hi < tile_kpos_lo) {
-            if ((p.flags & LTR_DKDV_BF16) && key_ok) {   // results, not accumulators: these keys get zeros
-                __bf16 *gz = p_role ? (__bf16 *)p.chunk[c].dv + b * p.dvs[0] + (long long)my_key * p.dvs[1] + hkv * p.dvs[2]
-                                    : (__bf16 *)p.chunk[c].dk + b * p.dks[0] + (long long)my_key * p.dks[1] + hkv * p.dks[2];
-                for (int d = 8 * hh; d < D; d += 16) *(uint4 *)(gz + d) = make_uint4(0, 0, 0, 0);
-            }
-            return;
-        }
-    }
-
-    // resident B operand: K rows for a P wave, V rows for a dS wave; lane (key l32, half hh) holds
-    // d = 16*kb + 8*hh .. +7
-    bf16x8 kvreg[D / 16];
-    {
-        const __bf16 *base = p_role ? (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2]
-                                    : (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
-        const long long rs = p_role ? p.ks[1] : p.vs[1];
-        const int ksafe = min(my_key, sk - 1);
-#pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) {
-            uint4 x = *(const uint4 *)(base + (long long)ksafe * rs + kb * 16 + 8 * hh);
-            if (!key_ok) x = make_uint4(0, 0, 0, 0);
-            kvreg[kb] = as_bf16x8(x);
-        }
-    }
-
-    f32x16 zero16;
-#pragma unroll
-    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
-    f32x16 acc[D / 32];                  // dV^T (P wave) or dK^T (dS wave)
-#pragma unroll
-    for (int i = 0; i < D / 32; i++) acc[i] = zero16;
-    const float c2 = p.scale * LTR_LOG2E;
-
-    // A tile's class depends on its rows only: 0 = no row sees any key of the block (skipped);
-    // 1 = every (row, key) pair is visible; 2 = needs the mask (diagonal, tails).
-    auto tile_class = [&](int qt) {
-        const int row0 = qt * BM;
-        const bool edge = key_tail || row0 + BM > p.Sq;
-        if (!causal) return edge ? 2 : 1;
-        int lo, hi;
-        q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
-        if (hi < tile_kpos_lo) return 0;
-        return (edge || tile_kpos_hi > lo) ? 2 : 1;
-    };
-
-    // The q tiles of each class are listed once per block (wave 0, ballot compaction: the order, and with it
-    // the rounding of the accumulation, is fixed), so the main loops carry no classification arithmetic.
-    unsigned short *const tlist = (unsigned short *)(smem + L::LIST_OFF);     // [2][MAX_QTILES]
-    int *const tcount = (int *)(smem + L::LIST_OFF + 2 * L::MAX_QTILES * 2);
-    if (w == 0) {
-        int n1 = 0, n2 = 0;
-        for (int base = 0; base < p.n_qtiles; base += 64) {
-            const int qt = base + lane;
-            const int cls = qt < p.n_qtiles ? tile_class(qt) : 0;
-            const unsigned long long m1 = __builtin_amdgcn_ballot_w64(cls == 1), m2 = __builtin_amdgcn_ballot_w64(cls == 2);
-            const unsigned long long below = (1ull << lane) - 1ull;
-            if (cls == 1) tlist[n1 + __builtin_popcountll(m1 & below)] = (unsigned short)qt;
-            if (cls == 2) tlist[L::MAX_QTILES + n2 + __builtin_popcountll(m2 & below)] = (unsigned short)qt;
-            n1 += __builtin_popcountll(m1);
-            n2 += __builtin_popcountll(m2);
-        }
-        if (lane == 0) {
-            tcount[0] = n1;
-            tcount[1] = n2;
-        }
-    }
-    __syncthreads();
-
-    const int st_row = lane / CPR, st_pc = lane % CPR;   // this lane's place inside a 1 KB LDS-direct load
-    const float st_mul = tid < BM ? -1.f / p.scale : -1.f;  // threads 0..63 stage -LSE/scale, 64..127 stage -DELTA
-    float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
-    bool sld_ok = true;
-    int sld_row0 = 0;     // first row of the tile in flight
-    unsigned *const pslot_base = (unsigned *)(smem + L::P_OFF) + slice * 4 * (L::P_SLOT / 4);
-
-    // two passes, each a loop of its own (unmasked tiles, then masked ones), so the accumulators
-    // live in straight-line loop bodies and the unmasked pass carries no bounds checks at all
-    auto run_pass = [&](auto mask_tag) {
-        constexpr bool MASK = decltype(mask_tag)::value;
-        constexpr int cls = MASK ? 2 : 1;
-        const int cnt = __builtin_amdgcn_readfirstlane(tcount[cls - 1]);
-        const unsigned short *const list = tlist + (cls - 1) * L::MAX_QTILES;
-        int li_ = -1;                                 // index into the list
-        // the list entry of the next call is read from LDS one call ahead, so its latency is never waited for
-        unsigned short pre = list[0];
-        auto advance = [&](int &rep, int &qt) {   // next tile of this class after (rep, qt); false when done
-            if (++li_ >= cnt) {
-                li_ = 0;
-                if (++rep >= p.n_rep) return false;
-            }
-            qt = __builtin_amdgcn_readfirstlane((int)pre);
-            pre = list[li_ + 1 < cnt ? li_ + 1 : 0];
-            return true;
-        };
-        // Q and dO tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane): wave w
-        // fills rows RPI*(NI*w + i) .. of both tiles with its i-th pair of loads, lane l the chunk position
-        // l % CPR of row l / CPR, fetching the logical chunk the swizzle places there.  Rows past the end of Q
-        // repeat its last row (they are masked).  LSE and DELTA go through a register of threads 0..127.
-        auto gload = [&](int rep, int qt, int buf) {
-            const int h = hkv * p.n_rep + rep;
-            const int row0 = qt * BM;
-            sld_row0 = row0;
-            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
-            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
-            const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
-            const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
-            const unsigned Qd = lds_address(smem) + buf * L::BUF_BYTES, dOd = Qd + L::TILE * 2;   // LDS byte addresses
-#pragma unroll
-            for (int i = 0; i < NI; i++) {
-                const int row = RPI * (NI * w + i) + st_row;
-                const int grow = MASK ? min(row0 + row, p.Sq - 1) : row0 + row;
-                const int chunk = st_pc ^ lds_swz<D>(row);
-                global_to_lds_b128(qp + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D * 2);
-                global_to_lds_b128(dop + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D * 2);
-            }
-            if (tid < 2 * BM) {
-                if (!MASK) {
-                    sld = sp[tid];
-                } else {
-                    const int r = tid < BM ? tid : tid - BM;
-                    sld_ok = row0 + r < p.Sq;
-                    sld = sp[sld_ok ? tid : (tid < BM ? 0 : BM)];
-                }
-            }
-        };
-        auto lds_store = [&](int buf) {   // the LSE / DELTA values fetched by gload
-            float *st = (float *)(smem + buf * L::BUF_BYTES) + L::TILE;   // after the two bf16 tiles
-            if (tid < 2 * BM) {
-                float x = sld * st_mul;
-                // rows past the end: -LSE/scale = -inf makes P = 0 (they are masked as well)
-                if (MASK) x = sld_ok ? x : (tid < BM ? -INFINITY : 0.f);
-                st[tid] = x;
-            } else if (MASK && tid < 3 * BM) {   // positions of the tile's rows (third wave)
-                const int row = sld_row0 + tid - 2 * BM;
-                ((int *)st)[tid] = row >= p.Sq ? BWD_QPOS_NONE
-                                   : causal ? q_position(row, p.q_split, p.q_pos0[0], p.q_pos0[1]) : BWD_QPOS_ALL;
-            }
-        };
-
-        const int kpos = key_ok ? pos0 + my_key : BWD_KPOS_NONE;
-        if (cnt == 0) return;
-        int rep = 0, qt = 0;
-        advance(rep, qt);
-        __syncthreads();   // the previous pass has finished reading LDS
-        gload(rep, qt, 0);
-        lds_store(0);
-        tile_barrier();
-        // One LDS barrier per 64-row tile.  In step t the P wave does all its work on tile t (S of both
-        // sub-tiles, P -> slots of parity t & 1, dV) and the dS wave all its work on tile t-1 (dP, dS with P
-        // from the slots filled one step earlier, dK): inside a step the two waves of a SIMD are independent,
-        // so one wave's softmax arithmetic runs under the other's MFMAs.  Slots of parity (t & 1) are
-        // rewritten in step t+2, after the barrier that ends step t+1 in which they were read.  Tile t+1 is
-        // fetched into registers at the start of step t and stored at its end into buffer (t+1) % 3, which
-        // held tile t-2, last read in step t-1.  Both roles execute T + 1 barriers.
-        auto put_slot = [&](unsigned *slot, const PackedTile &t) {
-            // two 16-byte halves per lane, each half contiguous over the lanes (no bank conflicts)
-            *(uint4 *)(slot + lane * 4) = make_uint4(t.u[0], t.u[1], t.u[2], t.u[3]);
-            *(uint4 *)(slot + 256 + lane * 4) = make_uint4(t.u[4], t.u[5], t.u[6], t.u[7]);
-        };
-        int par = 0;
-        // In the pass over unmasked tiles both loops are unrolled over the three Q / dO buffers (buf is a compile-time
-        // constant inside a step), so that LDS addresses are loop-invariant per-lane registers plus immediate offsets;
-        // the pass over masked tiles (few steps, more live registers) keeps one loop body with buf in a register.
-        if (p_role) {
-            bool more = true;
-            auto p_step = [&](auto buf_tag) {
-                const int buf = buf_tag;
-                more = advance(rep, qt);
-                const int nbuf = buf == L::NBUF - 1 ? 0 : buf + 1;
-                if (more) gload(rep, qt, nbuf);
-                const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
-                const __bf16 *dOs = Qs + L::TILE;
-                const float *st_s = (const float *)(dOs + L::TILE);   // -LSE/scale of the tile's rows
-                unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
-                // Accumulator register r of a sub-tile <-> tile row 8*(r/4) + 4*hh + r%4: both S accumulators start at
-                // -LSE/scale of their rows.  Order of the step: S of sub-tile a; S of sub-tile b with the
-                // exponentials of a issued under its MFMAs; first half of dV (rows of a) with the exponentials of b
-                // under its MFMAs; second half of dV.
-                f32x16 sa, sb;
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f32x4 la = *(const f32x4 *)(st_s + 8 * g + 4 * hh), lb = *(const f32x4 *)(st_s + 32 + 8 * g + 4 * hh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        sa[4 * g + e] = la[e];
-                        sb[4 * g + e] = lb[e];
-                    }
-                }
-                int qa[16], qb[16];   // positions of the rows (masked tiles only)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int *st_q = (const int *)st_s + 2 * BM;
-                    const i32x4 xa = MASK ? *(const i32x4 *)(st_q + 8 * g + 4 * hh) : i32x4{0, 0, 0, 0};
-                    const i32x4 xb = MASK ? *(const i32x4 *)(st_q + 32 + 8 * g + 4 * hh) : i32x4{0, 0, 0, 0};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        qa[4 * g + e] = xa[e];
-                        qb[4 * g + e] = xb[e];
-                    }
-                }
-                PackedTile ppa, ppb;
-                constexpr int NK = D / 16, ND = D / 32;
-                __builtin_amdgcn_s_setprio(1);
-                lds_gemm_chain<D>(Qs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, sa);
-                lds_gemm_chain<D>(Qs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, sb, [&](int kb) {
-#pragma unroll
-                    for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) ppa.u[j] = bwd_p_pair<MASK>(sa, j, c2, kpos, qa);
-                });
-                put_slot(slots, ppa);
-                bf16x8 pb[4];
-                pb[0] = operand_of(ppa, 0);
-                pb[1] = operand_of(ppa, 1);
-                // the operands of the second half do not exist yet: the hook below fills ppb while the first half
-                // runs, and the loop reads pb[2], pb[3] only after that; the first half reads pb[0], pb[1]
-                lds_tr_gemm<D, 2>(dOs, 0, lane, *(const bf16x8(*)[2]) & pb[0], acc, [&](int step) {
-#pragma unroll
-                    for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) ppb.u[j] = bwd_p_pair<MASK>(sb, j, c2, kpos, qb);
-                });
-                put_slot(slots + L::P_SLOT / 4, ppb);
-                pb[2] = operand_of(ppb, 0);
-                pb[3] = operand_of(ppb, 1);
-                lds_tr_gemm<D, 2>(dOs, 32, lane, *(const bf16x8(*)[2]) & pb[2], acc);
-                __builtin_amdgcn_s_setprio(0);
-                if (more) lds_store(nbuf);
-                tile_barrier();
-                par ^= 1;
-            };
-            static_assert(L::NBUF == 3, "unrolled over three buffers");
-            if (MASK) {
-                int buf = 0;
-                while (more) {
-                    p_step(buf);
-                    buf = buf == L::NBUF - 1 ? 0 : buf + 1;
-                }
-            } else {
-                for (;;) {
-                    p_step(std::integral_constant<int, 0>{});
-                    if (!more) break;
-                    p_step(std::integral_constant<int, 1>{});
-                    if (!more) break;
-                    p_step(std::integral_constant<int, 2>{});
-                    if (!more) break;
-                }
-            }
-            tile_barrier();                        // step T: only the dS waves have work
-        } else {
-            bool more = advance(rep, qt);          // step 0: staging duties only
-            if (more) gload(rep, qt, 1);
-            tile_barrier();
-            bool had_next = true;
-            auto ds_step = [&](auto buf_tag) {
-                const int buf = buf_tag;
-                had_next = more;
-                if (more) {
-                    more = advance(rep, qt);
-                    if (more) gload(rep, qt, buf + 2 >= L::NBUF ? buf + 2 - L::NBUF : buf + 2);
-                }
-                const __bf16 *Qs = (const __bf16 *)(smem + buf * L::BUF_BYTES);
-                const __bf16 *dOs = Qs + L::TILE;
-                const float *dlt_s = (const float *)(dOs + L::TILE) + BM;
-                const unsigned *slots = pslot_base + par * 2 * (L::P_SLOT / 4);
-                // the dP accumulators start at -DELTA of their rows (register r <-> tile row 8*(r/4) + 4*hh + r%4);
-                // same order as the P wave: dP of a; dP of b with dS of a under its MFMAs; first half of dK with dS of
-                // b under its MFMAs; second half of dK
-                f32x16 dpa, dpb;
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f32x4 da = *(const f32x4 *)(dlt_s + 8 * g + 4 * hh), db4 = *(const f32x4 *)(dlt_s + 32 + 8 * g + 4 * hh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        dpa[4 * g + e] = da[e];
-                        dpb[4 * g + e] = db4[e];
-                    }
-                }
-                PackedTile dsa, dsb;
-                constexpr int NK = D / 16, ND = D / 32;
-                __builtin_amdgcn_s_setprio(1);
-                lds_gemm_chain<D>(dOs + l32 * D, lds_swz<D>(l32) ^ hh, kvreg, dpa);
-                const uint4 pa0 = *(const uint4 *)(slots + lane * 4), pa1 = *(const uint4 *)(slots + 256 + lane * 4);
-                const unsigned pua[8] = {pa0.x, pa0.y, pa0.z, pa0.w, pa1.x, pa1.y, pa1.z, pa1.w};
-                lds_gemm_chain<D>(dOs + (32 + l32) * D, lds_swz<D>(32 + l32) ^ hh, kvreg, dpb, [&](int kb) {
-#pragma unroll
-                    for (int j = kb * (8 / NK); j < (kb + 1) * (8 / NK); j++) dsa.u[j] = bwd_ds_pair(pua[j], dpa, j);
-                });
-                const unsigned *slot_b = slots + L::P_SLOT / 4;
-                const uint4 pb0 = *(const uint4 *)(slot_b + lane * 4), pb1 = *(const uint4 *)(slot_b + 256 + lane * 4);
-                const unsigned pub[8] = {pb0.x, pb0.y, pb0.z, pb0.w, pb1.x, pb1.y, pb1.z, pb1.w};
-                bf16x8 db_[4];
-                db_[0] = operand_of(dsa, 0);
-                db_[1] = operand_of(dsa, 1);
-                lds_tr_gemm<D, 2>(Qs, 0, lane, *(const bf16x8(*)[2]) & db_[0], acc, [&](int step) {
-#pragma unroll
-                    for (int j = step * (4 / ND); j < (step + 1) * (4 / ND); j++) dsb.u[j] = bwd_ds_pair(pub[j], dpb, j);
-                });
-                db_[2] = operand_of(dsb, 0);
-                db_[3] = operand_of(dsb, 1);
-                lds_tr_gemm<D, 2>(Qs, 32, lane, *(const bf16x8(*)[2]) & db_[2], acc);
-                __builtin_amdgcn_s_setprio(0);
-                tile_barrier();
-                par ^= 1;
-            };
-            if (MASK) {
-                int buf = 0;
-                while (had_next) {
-                    ds_step(buf);
-                    buf = buf == L::NBUF - 1 ? 0 : buf + 1;
-                }
-            } else {
-                for (;;) {
-                    ds_step(std::integral_constant<int, 0>{});
-                    if (!had_next) break;
-                    ds_step(std::integral_constant<int, 1>{});
-                    if (!had_next) break;
-                    ds_step(std::integral_constant<int, 2>{});
-                    if (!had_next) break;
-                }
-            }
-        }
-    };
-    run_pass(std::false_type{});
-    run_pass(std::true_type{});
-
-    // dV^T (P wave) / dK^T (dS wave) tile of the wave's 32 keys: added to the fp32 accumulators in whole rows, through the
-    // wave's LDS staging area (every wave is past the last barrier: tiles, slots and lists are no longer read)
-    {
-        constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
-        const long long stride = uniform64(p_role ? p.dvs[1] : p.dks[1]);
-        const int key_base = uniform32(key0 + slice * 32), sk_u = uniform32(sk);
-        const long long goff = (p_role ? b * p.dvs[0] + hkv * p.dvs[2] : b * p.dks[0] + hkv * p.dks[2]) +
-                               (key_base + lane / LPR) * stride + 4 * (lane % LPR);
-        if (uniform32(p.flags & LTR_DKDV_BF16)) {   // every query that sees these keys was in this launch: store the result
-            __bf16 *gb = (__bf16 *)(p_role ? p.chunk[c].dv : p.chunk[c].dk) + goff;
-            wave_tile_rowmajor<D>(smem + w * WaveStage<D>::BYTES, lane, acc, p_role ? 1.f : p.scale, [&](int row, int, f32x4 val) {
-                if (key_base + row < sk_u) {
-                    bf16x4 y;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
-                    *(bf16x4 *)gb = y;
-                }
-                gb += ROWS_PER_IT * stride;
-            });
-            return;
-        }
-        float *gp = (p_role ? p.chunk[c].dv : p.chunk[c].dk) + goff;
-        // all reads of the accumulator first (independent loads in flight together), then the adds and the writes
-        constexpr int NIT = 32 / ROWS_PER_IT;
-        f32x4 old[NIT];
-#pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (key_base + it * ROWS_PER_IT + lane / LPR < sk_u) old[it] = *(const f32x4 *)(gp + it * ROWS_PER_IT * stride);
-        }
-        int it = 0;
-        wave_tile_rowmajor<D>(smem + w * WaveStage<D>::BYTES, lane, acc, p_role ? 1.f : p.scale, [&](int row, int, f32x4 val) {
-            if (key_base + row < sk_u) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) val[e] += old[it][e];
-                *(f32x4 *)gp = val;
-            }
-            gp += ROWS_PER_IT * stride;
-            it++;
-        });
-    }
 }
 
 // lds_gemm_chain / lds_tr_gemm for a wave that owns KW 32-key halves: every operand read from LDS feeds one MFMA per half
@@ -1469,30 +1056,9 @@ __device__ __forceinline__ void lds_tr_gemm_kw(const __bf16 *T, int row0, int la
     }
 }
 
-// LDS of bwd_dkdv_wide_kernel: as BwdLds with 256 keys per block (64 per wave pair) and twice the P slots
-template <int D>
-struct BwdLdsWide {
-    static constexpr int BN = 256;
-    static constexpr int BM = 64;
-    static constexpr int NT = 512;
-    static constexpr int TILE = BM * D;
-    static constexpr int BUF_BYTES = 2 * TILE * 2 + 3 * BM * 4;
-    static constexpr int P_SLOT = 64 * 32;
-    static constexpr int NBUF = 3;
-    static constexpr int P_OFF = NBUF * BUF_BYTES;
-    static constexpr int MAX_QTILES = 4096;
-    static constexpr int LIST_OFF = P_OFF + 4 * 4 * 2 * P_SLOT;           // 4 slices x 2 parities x 2 sub-tiles x 2 halves
-    static constexpr int TOTAL = LIST_OFF + 2 * MAX_QTILES * 2 + 16;
-    static_assert(TOTAL >= 8 * WaveStage<D>::BYTES, "the epilogue's staging areas reuse this memory");
-    static_assert(TOTAL <= 160 * 1024, "LDS of one CU");
-};
-
-// bwd_dkdv_kernel with two 32-key halves per wave (a block owns 256 keys): per MFMA half the LDS operand reads, half the
-// Q / dO transfers and half the per-step costs.  Fits the register file at head dim 64 only.
-template <int D>
-__global__ __launch_bounds__(512) void bwd_dkdv_wide_kernel(const BwdParams p) {
-    using L = BwdLdsWide<D>;
-    constexpr int KW = 2;   // 32-key halves per wave
+template <int D, int KW>
+__global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
+    using L = BwdLds<D, KW>;   // KW = 32-key halves per wave
     constexpr int BN = L::BN, BM = L::BM;
     constexpr int CPR = D / 8;
     constexpr int RPI = 64 / CPR;        // rows filled by one wave-wide LDS-direct load (1 KB)
@@ -1501,7 +1067,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_wide_kernel(const BwdParams p) {
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int slice = w & 3;             // 64-key slice; waves w and w+4 (same SIMD) are partners
+    const int slice = w & 3;             // slice of 32 * KW keys; waves w and w+4 (same SIMD) are partners
     const bool p_role = w < 4;           // P wave (S, P, dV) or dS wave (dP, dS, dK)
     const int l32 = lane & 31, hh = lane >> 5;
     const bool causal = p.flags & LTR_CAUSAL;
@@ -1948,273 +1514,6 @@ __global__ __launch_bounds__(512) void bwd_dkdv_wide_kernel(const BwdParams p) {
 // dQ: same block / wave / lane roles as the forward (a lane owns one query row), so LSE and DELTA are
 // per-lane scalars.  S^T = K Q^T and dP^T = V dO^T with K, V tiles natural in LDS; dS^T leaves the
 // registers as the B operand of dQ^T += K^T dS^T, whose A operand is the K tile read by transpose loads.
-template <int D>
-__global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
-    constexpr int NW = 8, BM = 32 * NW, BN = FwdTile<D>::BN;   // 8 waves (two per SIMD) share every K / V tile
-    constexpr int CPR = D / 8;
-    constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
-    constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // two {K tile, V tile} buffers,
-    constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
-    constexpr int BUF_ELEMS = 2 * TILE;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, hh = lane >> 5;
-    const bool causal = p.flags & LTR_CAUSAL;
-
-    int idx = blockIdx.x, pair, rest;
-    const int P = p.B * p.Hkv;
-    if ((P & 7) == 0) {
-        int xcd = idx & 7, j = idx >> 3, nr = p.n_slots * p.n_rep;
-        pair = (j / nr) * 8 + xcd;
-        rest = j % nr;
-    } else {
-        pair = idx % P;
-        rest = idx / P;
-    }
-    const int n_qt = (p.Sq + BM - 1) / BM;
-    const int rep = rest % p.n_rep, slot = rest / p.n_rep;
-    const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
-    // one q tile per block (late tiles first) or a late tile and its early counterpart (see q_tile_slots)
-    const bool paired = p.n_slots != n_qt;
-#pragma nounroll
-    for (int part = 0; part < 2; part++) {
-    const int qt = part == 0 ? n_qt - 1 - slot : slot;
-    if (part == 1 && (!paired || qt >= n_qt - 1 - slot)) break;
-    if (part == 1) __syncthreads();   // the first tile's epilogue used the LDS buffers as staging areas
-    int lane_of_part = threadIdx.x & 63;   // opaque per tile, see the forward kernel
-    asm volatile("" : "+v"(lane_of_part));
-    const int lane = lane_of_part, l32 = lane & 31, hh = lane >> 5;
-
-    const int row0 = qt * BM;
-    const int my_row = row0 + w * 32 + l32;
-    const bool row_ok = my_row < p.Sq;
-    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
-    int blk_lo, blk_hi, w_lo, w_hi;
-    q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
-    {
-        int wr0 = row0 + w * 32, wr1 = min(wr0 + 32, p.Sq) - 1;
-        if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
-        else { w_lo = -0x7fffffff; w_hi = -0x7fffffff; }  // wave has no valid row: everything masked
-    }
-
-    bf16x8 qreg[D / 16], doreg[D / 16];
-    float lse2 = INFINITY, dlt = 0.f;
-    {
-        const int rsafe = min(my_row, p.Sq - 1);
-        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + (long long)rsafe * p.qs[1] + h * p.qs[2];
-        const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + (long long)rsafe * p.dos[1] + h * p.dos[2];
-#pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) {
-            qreg[kb] = as_bf16x8(*(const uint4 *)(qp + kb * 16 + 8 * hh));
-            doreg[kb] = as_bf16x8(*(const uint4 *)(dop + kb * 16 + 8 * hh));
-        }
-        if (p.flags & LTR_DELTA_FROM_O) {
-            // DELTA = rowsum(dO * O) of this lane's row: its half of every 16-element block, then the other half's
-            const __bf16 *op = (const __bf16 *)p.o + b * p.os_[0] + (long long)rsafe * p.os_[1] + h * p.os_[2];
-            float part = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < D / 16; kb++) {
-                const bf16x8 ov = as_bf16x8(*(const uint4 *)(op + kb * 16 + 8 * hh));
-#pragma unroll
-                for (int e = 0; e < 8; e++) part += (float)ov[e] * (float)doreg[kb][e];
-            }
-            dlt = xhalf_sum(part);
-            if (row_ok && hh == 0) p.delta[((long long)b * p.Hq + h) * p.Sq + my_row] = dlt;
-        }
-        if (row_ok) {
-            // a row that saw no key has LSE = -inf: give it +inf like a row past the end, so that P = exp2(-inf) = 0
-            // whatever S is (S = -inf after the mask fix-up would otherwise meet -(-inf))
-            const float lse_row = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row];
-            lse2 = lse_row == -INFINITY ? INFINITY : lse_row * LTR_LOG2E;
-            if (!(p.flags & LTR_DELTA_FROM_O)) dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
-        }
-    }
-    f32x16 zero16;
-#pragma unroll
-    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
-    f32x16 dqacc[D / 32];
-#pragma unroll
-    for (int i = 0; i < D / 32; i++) dqacc[i] = zero16;
-    const float c2 = p.scale * LTR_LOG2E;
-
-    // The fields of the chunk being loaded live in scalar registers and are re-read from the argument
-    // table only when the chunk changes (a scalar load per tile would share the LDS wait counter).
-    int c = -1, t = 0, nt = 0;
-    int ld_sk = 0, ld_pos0 = 0;
-    const __bf16 *ld_kb = nullptr, *ld_vb = nullptr;
-    auto settle = [&]() {
-        while (c < p.n_chunks && t >= nt) {
-            c++;
-            t = 0;
-            if (c < p.n_chunks) {
-                ld_sk = p.chunk[c].sk;
-                ld_pos0 = p.chunk[c].pos0;
-                ld_kb = (const __bf16 *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
-                ld_vb = (const __bf16 *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
-                const int nvis = causal ? max(0, min(ld_sk, blk_hi - ld_pos0 + 1)) : ld_sk;
-                nt = (nvis + BN - 1) / BN;
-            }
-        }
-    };
-    settle();
-
-    // Tiles go from global memory straight into LDS (see the forward kernel): wave w fills rows
-    // RPI*(NI*w + i) .. with its i-th load; rows past the end of a chunk repeat its last row and are masked.
-    const int st_row = lane / CPR, st_pc = lane % CPR;
-    int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;   // the tile in flight: becomes the tile computed next
-    auto gload = [&](int ti, int buf) {
-        nx_sk = ld_sk;
-        nx_pos0 = ld_pos0;
-        nx_key0 = ti * BN;
-        const unsigned Kd = lds_address(smem) + buf * BUF_ELEMS * 2, Vd = Kd + TILE * 2;   // LDS byte addresses
-#pragma unroll
-        for (int i = 0; i < NI; i++) {
-            const int row = RPI * (NI * w + i) + st_row;
-            const int key = min(ti * BN + row, ld_sk - 1);
-            const int chunk = st_pc ^ lds_swz<D>(row);
-            global_to_lds_b128(ld_kb + (long long)(key * (int)p.ks[1] + chunk * 8), Kd + RPI * (NI * w + i) * D * 2);
-            global_to_lds_b128(ld_vb + (long long)(key * (int)p.vs[1] + chunk * 8), Vd + RPI * (NI * w + i) * D * 2);
-        }
-    };
-
-    bool have = c < p.n_chunks;
-    if (have) gload(t, 0);
-    tile_barrier();
-    // LDS byte addresses of this lane's operands in the K tile of the current buffer (the V tile and the other 32-key
-    // blocks are immediates away): kept in registers and flipped to the other buffer with one XOR each per tile
-    static_assert((BUF_ELEMS * 2 & (BUF_ELEMS * 2 - 1)) == 0, "buffer size must be a power of two for the XOR flip");
-    unsigned pa[D / 16], ta[D / 32][2];
-    {
-        const unsigned lds0 = lds_address(smem);   // the only LDS object of the kernel: aligned far beyond the buffer size
-        const int sw = lds_swz<D>(l32) ^ hh;        // rows l32 + 32 n share the swizzle word of row l32
-#pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) pa[kb] = lds0 + ((l32 * D + (((2 * kb) ^ sw) << 3)) << 1);
-        const int li = lane & 15, g = lane >> 4;
-#pragma unroll
-        for (int j = 0; j < D / 32; j++)
-#pragma unroll
-            for (int e = 0; e < 2; e++) {
-                const int col = j * 32 + ((g & 1) << 4) + ((li & 3) << 2), row = 4 * (g >> 1) + (li >> 2) + 8 * e;
-                ta[j][e] = lds0 + ((lds_swz_off<D>(row, col >> 3) + (col & 7)) << 1);
-            }
-    }
-    int par = 0;
-    while (have) {
-        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0;
-        t++;
-        settle();
-        const bool have_next = c < p.n_chunks;
-        if (have_next) gload(t, par ^ 1);
-
-        const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
-        // 32 keys at a time, one block after the other: one live (S^T, dP^T) tile pair keeps the kernel at two
-        // waves per SIMD, and the other wave's MFMAs cover this wave's softmax arithmetic.  A wave whose rows all
-        // precede the tile's first key has nothing to add (see the forward kernel).
-        if (!causal || pos0 + key0 <= w_hi) {
-#pragma unroll
-        for (int nb = 0; nb < BN / 32; nb++) {
-            f32x16 s = zero16, dp = zero16;
-            __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
-            lds_gemm_pair_at<D>(pa, nb * 32 * D * 2, TILE * 2 + nb * 32 * D * 2, qreg, doreg, s, dp);
-            __builtin_amdgcn_s_setprio(0);
-            // mask fix-up (tail of the chunk, diagonal tiles, rows past the end): wave-uniform branch touching S only;
-            // an invisible entry gets S = -inf, so P = 0 and dS = 0
-            if (need_mask) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
-                    const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
-                    s[r] = vis ? s[r] : -INFINITY;
-                }
-            }
-            PackedTile ds;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                float dsv[2];
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int r = 2 * j + e;
-                    const float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2);
-                    dsv[e] = pv * (dp[r] - dlt);
-                }
-                ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
-            }
-            __builtin_amdgcn_s_setprio(1);
-            {
-                const bf16x8 dsb[2] = {operand_of(ds, 0), operand_of(ds, 1)};
-                lds_tr_gemm_at<D, 2>(ta, nb * 32 * D * 2, dsb, dqacc);   // 16 keys per MFMA
-            }
-            __builtin_amdgcn_s_setprio(0);
-        }
-        }
-        tile_barrier();
-#pragma unroll
-        for (int kb = 0; kb < D / 16; kb++) pa[kb] ^= BUF_ELEMS * 2;
-#pragma unroll
-        for (int j = 0; j < D / 32; j++) {
-            ta[j][0] ^= BUF_ELEMS * 2;
-            ta[j][1] ^= BUF_ELEMS * 2;
-        }
-        par ^= 1;
-        have = have_next;
-    }
-
-    // dQ in whole rows through the wave's LDS staging area (the tiles are no longer read: the last barrier is behind us)
-    {
-        constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
-        unsigned char *stage = smem + w * WaveStage<D>::BYTES;
-        const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + w * 32);
-        const long long dqs1 = uniform64(p.dqs[1]);
-        const long long off0 = uniform64(b * p.dqs[0] + h * p.dqs[2]) + (wave_row0 + lane / LPR) * dqs1 + 4 * (lane % LPR);
-        // LTR_ROPE_DQ: q was rotated by the forward's prologue, so the gradient of the caller's un-rotated q is dQ rotated by
-        // the conjugate angles of its row's position (the rotation is linear: it commutes with the accumulation over calls)
-        const bool rope = uniform32(p.flags & LTR_ROPE_DQ) != 0;
-        const float *const rope_tab = p.rope;
-        const int rope_p0 = uniform32(p.rope_pos0), split_u = uniform32(p.q_split), qp0 = uniform32(p.q_pos0[0]), qp1 = uniform32(p.q_pos0[1]);
-        auto unrotate = [&](int row, int col, f32x4 val) {
-            if (!rope) return val;
-            const int pos = q_position(wave_row0 + row, split_u, qp0, qp1);
-            return rope_conj4(val, *(const f32x4 *)(rope_tab + (long long)(pos - rope_p0) * D + col));
-        };
-        if (uniform32(p.flags & LTR_DQ_BF16)) {   // this call saw every key of these rows: store the result, no accumulator
-            __bf16 *dqp = (__bf16 *)p.dq + off0;
-            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int col, f32x4 val) {
-                if (wave_row0 + row < Sq_u) {
-                    val = unrotate(row, col, val);
-                    bf16x4 y;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) y[e] = (__bf16)val[e];
-                    *(bf16x4 *)dqp = y;
-                }
-                dqp += ROWS_PER_IT * dqs1;
-            });
-        } else {
-            float *dqp = (float *)p.dq + off0;
-            constexpr int NIT = 32 / ROWS_PER_IT;
-            f32x4 old[NIT];   // all reads of the accumulator first, then the adds and the writes
-#pragma unroll
-            for (int it = 0; it < NIT; it++) {
-                old[it] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (wave_row0 + it * ROWS_PER_IT + lane / LPR < Sq_u) old[it] = *(const f32x4 *)(dqp + it * ROWS_PER_IT * dqs1);
-            }
-            int it = 0;
-            wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int col, f32x4 val) {
-                if (wave_row0 + row < Sq_u) {
-                    val = unrotate(row, col, val);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) val[e] += old[it][e];
-                    *(f32x4 *)dqp = val;
-                }
-                dqp += ROWS_PER_IT * dqs1;
-                it++;
-            });
-        }
-    }
-    }   // part
-}
-
 // lds_gemm_pair_at / lds_tr_gemm_at for a wave that owns RB 32-row blocks: every operand read from LDS feeds one MFMA per row
 // block (ba[rb], bb[rb], ra[rb], rb_[rb] / b[rb], acc[rb] belong to row block rb).
 template <int D, int RB>
@@ -2270,11 +1569,8 @@ __device__ __forceinline__ void lds_tr_gemm_at_rb(const unsigned (&addr)[D / 32]
     }
 }
 
-// bwd_dq_kernel with two 32-row blocks per wave (a block owns 512 query rows, a lane two of them): per MFMA half the LDS
-// operand reads, half the K / V transfers and half the per-tile costs.  Fits the register file at head dim 64 only.
-template <int D>
-__global__ __launch_bounds__(512) void bwd_dq_wide_kernel(const BwdParams p) {
-    constexpr int RB = 2;   // 32-row blocks per wave: a lane owns RB query rows
+template <int D, int RB>   // RB = 32-row blocks per wave: a lane owns RB query rows, a block 256 * RB
+__global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     constexpr int NW = 8, BM = 32 * RB * NW, BN = FwdTile<D>::BN;   // 8 waves (two per SIMD) share every K / V tile
     constexpr int CPR = D / 8;
     constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
@@ -2806,21 +2102,21 @@ int enable_large_lds() {
     int dev = 0;
     if (current_device(&dev)) return LTR_EDEVICE;
     if (g_dev[dev].large_lds.load(std::memory_order_acquire) == 1) return LTR_OK;
-    bool ok = hipFuncSetAttribute((const void *)bwd_dkdv_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  BwdLds<128>::TOTAL) == hipSuccess &&
-              hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  BwdLds<64>::TOTAL) == hipSuccess &&
-              hipFuncSetAttribute((const void *)bwd_dkdv_wide_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  BwdLdsWide<64>::TOTAL) == hipSuccess &&
+    bool ok = hipFuncSetAttribute((const void *)bwd_dkdv_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  BwdLds<128, 1>::TOTAL) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  BwdLds<64, 1>::TOTAL) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  BwdLds<64, 2>::TOTAL) == hipSuccess &&
               hipFuncSetAttribute((const void *)fwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   fwd_lds_bytes<128>()) == hipSuccess &&
               hipFuncSetAttribute((const void *)fwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   fwd_lds_bytes<64>()) == hipSuccess &&
-              hipFuncSetAttribute((const void *)bwd_dq_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+              hipFuncSetAttribute((const void *)bwd_dq_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<128>()) == hipSuccess &&
-              hipFuncSetAttribute((const void *)bwd_dq_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+              hipFuncSetAttribute((const void *)bwd_dq_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<64>()) == hipSuccess &&
-              hipFuncSetAttribute((const void *)bwd_dq_wide_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+              hipFuncSetAttribute((const void *)bwd_dq_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<64>()) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
@@ -3059,7 +2355,7 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     if (do_dq && !strides_ok(a->dq_stride, (flags & LTR_DQ_BF16) ? 2 : 4)) return LTR_EALIGN;
     if (fused_delta && (!aligned16(a->o) || !strides_ok(a->o_stride, 2))) return LTR_EALIGN;
     if (fused_delta && (a->Sq + 64) * a->o_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
-    if ((a->Sq + 63) / 64 > BwdLds<128>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
+    if ((a->Sq + 63) / 64 > BwdLds<128, 1>::MAX_QTILES) return LTR_EUNSUP;       // q tile lists live in LDS
     if ((a->Sq + 64) * a->q_stride[1] >= 0x7fffffffLL || (a->Sq + 64) * a->do_stride[1] >= 0x7fffffffLL) return LTR_EUNSUP;
     BwdParams p;
     p.rope = nullptr;
@@ -3087,7 +2383,7 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         if (cus <= 0) cus = 256;
         wide = steps >= 48 && blocks256 >= (long long)((flags & LTR_CAUSAL) ? 4 : 2) * cus;
     }
-    const int keys_per_block = wide ? BwdLdsWide<64>::BN : 128;
+    const int keys_per_block = wide ? BwdLds<64, 2>::BN : BwdLds<64, 1>::BN;
     long long tiles = 0;
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];
@@ -3186,9 +2482,9 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     const long long nblk_q = (long long)p.n_slots * p.B * p.Hq;
     // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
     if (do_dq) {
-        if (a->D == 128) hipLaunchKernelGGL(bwd_dq_kernel<128>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
-        else if (wide_q) hipLaunchKernelGGL(bwd_dq_wide_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
-        else hipLaunchKernelGGL(bwd_dq_kernel<64>, dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
+        if (a->D == 128) hipLaunchKernelGGL((bwd_dq_kernel<128, 1>), dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
+        else if (wide_q) hipLaunchKernelGGL((bwd_dq_kernel<64, 2>), dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
+        else hipLaunchKernelGGL((bwd_dq_kernel<64, 1>), dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
     }
     if (do_dkdv) {
         // A block of the dK/dV kernel owns 128 keys and loops over the query tiles that see them: under a causal mask its
@@ -3197,9 +2493,9 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         // the tail (the sums inside a block do not depend on the table's order).
         if (flags & LTR_CAUSAL)
             std::stable_sort(p.chunk, p.chunk + p.n_chunks, [](const ChunkDev &x, const ChunkDev &y) { return x.pos0 < y.pos0; });
-        if (a->D == 128) hipLaunchKernelGGL(bwd_dkdv_kernel<128>, dim3((unsigned)nblk), dim3(BwdLds<128>::NT), BwdLds<128>::TOTAL, st, p);
-        else if (wide) hipLaunchKernelGGL(bwd_dkdv_wide_kernel<64>, dim3((unsigned)nblk), dim3(BwdLdsWide<64>::NT), BwdLdsWide<64>::TOTAL, st, p);
-        else hipLaunchKernelGGL(bwd_dkdv_kernel<64>, dim3((unsigned)nblk), dim3(BwdLds<64>::NT), BwdLds<64>::TOTAL, st, p);
+        if (a->D == 128) hipLaunchKernelGGL((bwd_dkdv_kernel<128, 1>), dim3((unsigned)nblk), dim3(BwdLds<128, 1>::NT), (BwdLds<128, 1>::TOTAL), st, p);
+        else if (wide) hipLaunchKernelGGL((bwd_dkdv_kernel<64, 2>), dim3((unsigned)nblk), dim3(BwdLds<64, 2>::NT), (BwdLds<64, 2>::TOTAL), st, p);
+        else hipLaunchKernelGGL((bwd_dkdv_kernel<64, 1>), dim3((unsigned)nblk), dim3(BwdLds<64, 1>::NT), (BwdLds<64, 1>::TOTAL), st, p);
     }
     return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }
