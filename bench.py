@@ -335,7 +335,8 @@ def _run_attention(la, torch, cfg, steps, warmup, data="randn"):
         kernels["bwd_dq_kernel"] = {"ms_per_launch": round(dq_ms, 4), "gemms_credited": 1, "gemms_executed": 3,
                                     "algorithmic_tflops": round(0.5 * f_share / dq_ms / 1e9, 2),
                                     "executed_tflops": round(1.5 * f_share / dq_ms / 1e9, 2)}
-        dom, dom_ms, dom_flops = "bwd_dkdv_kernel<%d>" % D, dkdv_ms, 2.0 * f_share
+        # template arguments: head dim, 32-key halves per wave (2 = the 256-key blocks the library picks for long head-dim-64 streams)
+        dom, dom_ms, dom_flops = "bwd_dkdv_kernel<%d, %d>" % (D, 2 if (D == 64 and not causal and S >= 4096) else 1), dkdv_ms, 2.0 * f_share
     else:
         dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_share
     return {"dt": dt, "f_total": f_total, "kernels": kernels, "launches": launches,

@@ -133,18 +133,18 @@ def test_bench_traffic_figure_is_tied_to_the_kernel_source(tmp_path, monkeypatch
     src.write_text("kernel text")
     prof = tmp_path / "counters.md"
     digest = hashlib.sha256(src.read_bytes()).hexdigest()
-    prof.write_text("x\nkernel-source-sha256: %s\ntraffic-bytes-per-launch bwd_dkdv_kernel<128>: 1.2988e+09\n" % digest)
+    prof.write_text("x\nkernel-source-sha256: %s\ntraffic-bytes-per-launch bwd_dkdv_kernel<128, 1>: 1.2988e+09\n" % digest)
     monkeypatch.setattr(bench, "KERNEL_SOURCE", str(src))
     monkeypatch.setattr(bench, "COUNTER_PROFILE", str(prof))
-    val, why = bench._measured_traffic("bwd_dkdv_kernel<128>")
+    val, why = bench._measured_traffic("bwd_dkdv_kernel<128, 1>")
     assert val == 1.2988e9 and digest[:12] in why
     assert bench._measured_traffic("fwd_bf16_kernel<128>")[0] is None      # no line for that kernel
     src.write_text("kernel text, edited")
-    val, why = bench._measured_traffic("bwd_dkdv_kernel<128>")
+    val, why = bench._measured_traffic("bwd_dkdv_kernel<128, 1>")
     assert val is None and "stale" in why
     # the committed profile and the committed source: either in step (a number) or flagged, never an exception
     monkeypatch.undo()
-    val, why = bench._measured_traffic("bwd_dkdv_kernel<128>")
+    val, why = bench._measured_traffic("bwd_dkdv_kernel<128, 1>")
     assert (val is None) or val > 0
 
 
