@@ -259,3 +259,42 @@ def test_config5_full_ulysses_layout(ltr):
     _check_keys(qf, kf, vf, oc, lsec, dof, pos, pos, False, dk_h, dv_h, n=6)
     # heads outside group r received no gradient
     assert qd.grad[0][:, :, :r * (H // W)].abs().max() == 0
+
+
+@pytest.mark.parametrize("keys,rows", [(256, 512), (128, 256)])
+def test_head_dim_64_ring_share_both_block_sizes(ltr, keys, rows):
+    """Head dim 64 at a size where the 256-key dK/dV blocks and 512-row dQ blocks are what the library runs: one zig-zag rank
+    share (rank 2 of 4: half-chunks 2 and 5 of 8 x 2048 positions) of a causal GQA 8/2 sequence of 16384, B = 2, against all
+    8 KV half-chunks in ring order, fp32 dK / dV accumulators, bf16 dQ with DELTA from O.  Both block sizes forced through
+    the hint flags; sampled rows (O, LSE, dQ) and sampled keys (dK, dV) against the oracle's closed form."""
+    g = torch.Generator().manual_seed(5)
+    B, Hq, Hkv, D, S, W = 2, 8, 2, 64, 16384, 4
+    hc = S // (2 * W)
+    q = torch.randn(B, S, Hq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+    r = 2
+    qpos = orc.zigzag_positions(r, W, S)
+    do = torch.randn(B, 2 * hc, Hq, D, generator=g).to(torch.bfloat16)
+    kd, vd = k.cuda(), v.cuda()
+    ql, dol = q[:, qpos].cuda(), do.cuda()
+    order = []
+    for j in orc.ring_order(r, W):
+        order += [j, 2 * W - 1 - j]                      # the two half-chunks of rank j
+    ks = [kd[:, i * hc:(i + 1) * hc] for i in order]
+    vs = [vd[:, i * hc:(i + 1) * hc] for i in order]
+    pos0 = [i * hc for i in order]
+    qp = (r * hc, (2 * W - 1 - r) * hc)
+    ol, lsel = ltr.attn_fwd(ql, ks, vs, pos0, qp, hc, True)
+    dk = torch.zeros(kd.shape, dtype=torch.float32, device="cuda")
+    dv = torch.zeros(vd.shape, dtype=torch.float32, device="cuda")
+    dks = [dk[:, i * hc:(i + 1) * hc] for i in order]
+    dvs = [dv[:, i * hc:(i + 1) * hc] for i in order]
+    dq = torch.empty(ql.shape, dtype=torch.bfloat16, device="cuda")
+    delta_ws = torch.empty(B, Hq, 2 * hc, dtype=torch.float32, device="cuda")
+    ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, qp, hc, True, do_dkdv=False, o=ol, dq_rows=rows)
+    ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, qp, hc, True, do_dq=False, dkdv_keys=keys)
+    kpos = torch.arange(S)
+    oc, lsec = ol.cpu(), lsel.cpu()
+    _check_rows(q[:, qpos], k, v, qpos, kpos, True, oc, lsec, do, dq.cpu(), n=20)
+    _check_keys(q[:, qpos], k, v, oc, lsec, do, qpos, kpos, True, dk.cpu(), dv.cpu(), n=8)
