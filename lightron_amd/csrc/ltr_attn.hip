@@ -473,9 +473,8 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
     constexpr int BUF_ELEMS = 2 * TILE;
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, hh = lane >> 5;
     const bool causal = p.flags & LTR_CAUSAL;
 
     // block -> (batch, kv head, q head of the group, q tile).  Consecutive block ids go to
@@ -1579,9 +1578,8 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     constexpr int TILE = BN * D;             // rows unpadded, 16-byte chunks XOR-swizzled (lds_swz)
     constexpr int BUF_ELEMS = 2 * TILE;
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, hh = lane >> 5;
     const bool causal = p.flags & LTR_CAUSAL;
 
     int idx = blockIdx.x, pair, rest;
@@ -2135,15 +2133,20 @@ bool strides_ok(const int64_t *s, int elem_bytes) {
 
 int fits_i32(int64_t x) { return x >= 0 && x < (int64_t)0x7fffffff; }
 
+// compute units of the current device (the launch heuristics below count rounds of blocks over them)
+int device_cus() {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    return cus > 0 ? cus : 256;
+}
+
 // Slots of q tiles handed to the blocks of the forward and dQ kernels.  Under a causal mask a tile's work grows with its
 // rows' positions; pairing tile t with tile n - 1 - t in one block gives every block the same work (no long blocks left
 // over at the end of the launch) and halves the number of blocks to start.  Only done while the equal blocks still fill
 // the device's CUs evenly; otherwise one tile per slot, heaviest first, and the hardware's in-order dispatch balances.
 int q_tile_slots(int n_qtiles, long long blocks_per_tile, bool causal) {
     if (!causal || n_qtiles < 2) return n_qtiles;
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (cus <= 0) cus = 256;
+    const int cus = device_cus();
     const int n_slots = (n_qtiles + 1) / 2;
     const long long n = n_slots * blocks_per_tile, rounds = (n + cus - 1) / cus;
     return n * 10 >= rounds * cus * 9 ? n_slots : n_qtiles;
@@ -2378,9 +2381,7 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         for (int c = 0; c < a->n_chunks; c++) blocks256 += (a->chunk[c].sk + 255) / 256;
         blocks256 *= (long long)a->B * a->Hkv;
         const long long steps = (long long)(a->Hq / a->Hkv) * ((a->Sq + 63) / 64) / ((flags & LTR_CAUSAL) ? 2 : 1);
-        int dev = 0, cus = 256;
-        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        if (cus <= 0) cus = 256;
+        const int cus = device_cus();
         wide = steps >= 48 && blocks256 >= (long long)((flags & LTR_CAUSAL) ? 4 : 2) * cus;
     }
     const int keys_per_block = wide ? BwdLds<64, 2>::BN : BwdLds<64, 1>::BN;
@@ -2471,9 +2472,7 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         const bool causal_ = (flags & LTR_CAUSAL) != 0;
         const int tiles512 = (p.Sq + 511) / 512, slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_);
         const long long blocks512 = (long long)slots512 * p.B * p.Hq;
-        int dev = 0, cus = 256;
-        if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        if (cus <= 0) cus = 256;
+        const int cus = device_cus();
         // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance
         wide_q = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus) : (blocks512 * 4 >= (long long)cus * 3);
     }
