@@ -2140,12 +2140,35 @@ int device_cus() {
     return cus > 0 ? cus : 256;
 }
 
+// Keys that the q rows [r0, r1] walk through under the causal mask: per chunk, those up to the rows' last position.
+long long visible_keys(int r0, int r1, int q_split, const int *q_pos0, const ChunkDev *chunk, int n_chunks) {
+    auto pos = [&](int row) { return row < q_split ? q_pos0[0] + row : q_pos0[1] + (row - q_split); };
+    int hi = pos(r1);
+    if (r0 < q_split && r1 >= q_split) hi = std::max(hi, pos(q_split - 1));
+    long long keys = 0;
+    for (int c = 0; c < n_chunks; c++) keys += std::min<long long>(std::max<long long>((long long)hi - chunk[c].pos0 + 1, 0), chunk[c].sk);
+    return keys;
+}
+
+// Under a causal mask, do the q tiles of `rows` rows differ in work?  Compared are the first and the last tile: a late
+// chunk of a long ring sees nearly all keys from every tile (nothing to balance), a single causal chunk 1 / n of them
+// from its first tile.
+bool q_tiles_uneven(int Sq, int rows, int q_split, const int *q_pos0, const ChunkDev *chunk, int n_chunks) {
+    const int n = (Sq + rows - 1) / rows;
+    if (n < 2) return false;
+    const long long first = visible_keys(0, rows - 1, q_split, q_pos0, chunk, n_chunks);
+    const long long last = visible_keys((n - 1) * rows, Sq - 1, q_split, q_pos0, chunk, n_chunks);
+    return std::min(first, last) * 4 < std::max(first, last) * 3;
+}
+
 // Slots of q tiles handed to the blocks of the forward and dQ kernels.  Under a causal mask a tile's work grows with its
 // rows' positions; pairing tile t with tile n - 1 - t in one block gives every block the same work (no long blocks left
-// over at the end of the launch) and halves the number of blocks to start.  Only done while the equal blocks still fill
-// the device's CUs evenly; otherwise one tile per slot, heaviest first, and the hardware's in-order dispatch balances.
-int q_tile_slots(int n_qtiles, long long blocks_per_tile, bool causal) {
-    if (!causal || n_qtiles < 2) return n_qtiles;
+// over at the end of the launch) and halves the number of blocks to start.  Only done when the tiles do differ (see
+// q_tiles_uneven: paired tiles run one after the other, so fewer blocks walk through the same K / V rows at the same time)
+// and while the equal blocks still fill the device's CUs evenly; otherwise one tile per slot, heaviest first, and the
+// hardware's in-order dispatch balances.
+int q_tile_slots(int n_qtiles, long long blocks_per_tile, bool uneven) {
+    if (!uneven || n_qtiles < 2) return n_qtiles;
     const int cus = device_cus();
     const int n_slots = (n_qtiles + 1) / 2;
     const long long n = n_slots * blocks_per_tile, rounds = (n + cus - 1) / cus;
@@ -2275,7 +2298,8 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     if (a->io_dtype == LTR_BF16) {
         p.n_qtiles = (p.Sq + 255) / 256;
         if ((long long)p.n_qtiles * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
-        p.n_slots = q_tile_slots(p.n_qtiles, (long long)p.B * p.Hq, (p.flags & LTR_CAUSAL) != 0);
+        p.n_slots = q_tile_slots(p.n_qtiles, (long long)p.B * p.Hq,
+                                 (p.flags & LTR_CAUSAL) && q_tiles_uneven(p.Sq, 256, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
         const long long nblk = (long long)p.n_slots * p.B * p.Hq;
         rc = enable_large_lds();
         if (rc) return rc;
@@ -2470,14 +2494,16 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         wide_q = true;
     } else if (!(flags & LTR_DQ_ROWS_256) && a->D == 64 && do_dq) {
         const bool causal_ = (flags & LTR_CAUSAL) != 0;
-        const int tiles512 = (p.Sq + 511) / 512, slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_);
+        const int tiles512 = (p.Sq + 511) / 512;
+        const int slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_ && q_tiles_uneven(p.Sq, 512, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
         const long long blocks512 = (long long)slots512 * p.B * p.Hq;
         const int cus = device_cus();
         // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance
         wide_q = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus) : (blocks512 * 4 >= (long long)cus * 3);
     }
     const int dq_rows = wide_q ? 512 : 256;
-    p.n_slots = q_tile_slots((p.Sq + dq_rows - 1) / dq_rows, (long long)p.B * p.Hq, (flags & LTR_CAUSAL) != 0);
+    p.n_slots = q_tile_slots((p.Sq + dq_rows - 1) / dq_rows, (long long)p.B * p.Hq,
+                             (flags & LTR_CAUSAL) && q_tiles_uneven(p.Sq, dq_rows, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
     const long long nblk_q = (long long)p.n_slots * p.B * p.Hq;
     // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
     if (do_dq) {
