@@ -2133,6 +2133,12 @@ bool strides_ok(const int64_t *s, int elem_bytes) {
 
 int fits_i32(int64_t x) { return x >= 0 && x < (int64_t)0x7fffffff; }
 
+// How evenly `blocks` equal blocks, one per CU at a time, fill the CUs: blocks / (rounds x CUs), 1 = no idle CU in any round.
+double cu_fill(long long blocks, int cus) {
+    const long long rounds = (blocks + cus - 1) / cus;
+    return rounds > 0 ? (double)blocks / (double)(rounds * cus) : 0.0;
+}
+
 // compute units of the current device (the launch heuristics below count rounds of blocks over them)
 int device_cus() {
     int dev = 0, cus = 256;
@@ -2394,19 +2400,26 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         p.rope = a->rope_freqs;
         p.rope_pos0 = (int)a->rope_pos0;
     }
-    // keys per block of the dK/dV kernel: 256 (two 32-key halves per wave) pays at head dim 64 when a block walks many q tiles
-    // and the wider blocks still fill the device several times over; the caller can force either size
+    // keys per block of the dK/dV kernel: 256 (two 32-key halves per wave, about 12 % less time per key) pays at head dim 64
+    // when the wider blocks fill the device's CUs about as evenly as the 128-key blocks do (equal blocks, no mask), or, under
+    // a causal mask (unequal blocks), when a block walks many q tiles and there are several rounds of blocks to balance
+    // with; the caller can force either size
     bool wide = false;
     if (flags & LTR_DKDV_KEYS_256) {
         if (a->D != 64 || f32) return LTR_EUNSUP;
         wide = true;
     } else if (!(flags & LTR_DKDV_KEYS_128) && a->D == 64 && !f32 && do_dkdv) {
-        long long blocks256 = 0;
-        for (int c = 0; c < a->n_chunks; c++) blocks256 += (a->chunk[c].sk + 255) / 256;
+        long long blocks256 = 0, blocks128 = 0;
+        for (int c = 0; c < a->n_chunks; c++) {
+            blocks256 += (a->chunk[c].sk + 255) / 256;
+            blocks128 += (a->chunk[c].sk + 127) / 128;
+        }
         blocks256 *= (long long)a->B * a->Hkv;
-        const long long steps = (long long)(a->Hq / a->Hkv) * ((a->Sq + 63) / 64) / ((flags & LTR_CAUSAL) ? 2 : 1);
+        blocks128 *= (long long)a->B * a->Hkv;
+        const long long q_tiles = (long long)(a->Hq / a->Hkv) * ((a->Sq + 63) / 64);
         const int cus = device_cus();
-        wide = steps >= 48 && blocks256 >= (long long)((flags & LTR_CAUSAL) ? 4 : 2) * cus;
+        if (flags & LTR_CAUSAL) wide = q_tiles >= 96 && blocks256 >= 4LL * cus;
+        else wide = q_tiles >= 16 && cu_fill(blocks256, cus) * 1.12 >= cu_fill(blocks128, cus);
     }
     const int keys_per_block = wide ? BwdLds<64, 2>::BN : BwdLds<64, 1>::BN;
     long long tiles = 0;
@@ -2498,8 +2511,11 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         const int slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_ && q_tiles_uneven(p.Sq, 512, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
         const long long blocks512 = (long long)slots512 * p.B * p.Hq;
         const int cus = device_cus();
-        // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance
-        wide_q = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus) : (blocks512 * 4 >= (long long)cus * 3);
+        // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance; no mask: the wider
+        // blocks (about 7 % less time per row) must fill the CUs about as evenly as the 256-row blocks
+        const long long blocks256 = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
+        wide_q = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus)
+                         : (cu_fill(blocks512, cus) * 1.07 >= cu_fill(blocks256, cus));
     }
     const int dq_rows = wide_q ? 512 : 256;
     p.n_slots = q_tile_slots((p.Sq + dq_rows - 1) / dq_rows, (long long)p.B * p.Hq,
