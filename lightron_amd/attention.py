@@ -28,7 +28,7 @@ def _s3(t: torch.Tensor):
 def _req(t: torch.Tensor, name: str):
     if not t.is_cuda:
         raise RuntimeError("%s must be a GPU tensor (the HIP library has no CPU path)" % name)
-    if t.dim() != 4 or t.stride(3) != 1:
+    if t.dim() != 4 or (t.numel() > 0 and t.stride(3) != 1):
         raise RuntimeError("%s must be [B,S,H,D] with a contiguous last dim, got shape %s strides %s"
                            % (name, tuple(t.shape), t.stride()))
 
@@ -99,6 +99,8 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
     _req(out, "out")
     if lse is None or lse.dtype != torch.float32 or not lse.is_contiguous() or tuple(lse.shape) != (B, Hq, Sq):
         raise RuntimeError("lse must be a contiguous fp32 [B,Hq,Sq] tensor")
+    if q.numel() == 0:          # no query rows: the reference's matmuls return an empty result as well
+        return out, lse
     a = _lib.FwdArgs()
     a.q, a.o, a.lse = q.data_ptr(), out.data_ptr(), lse.data_ptr()
     a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, Hkv, D, Sq
@@ -140,6 +142,8 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
     _req(do, "dO")
     B, Sq, Hq, D = o.shape
     delta = torch.empty((B, Hq, Sq), dtype=torch.float32, device=o.device)
+    if o.numel() == 0:
+        return delta
     a = _lib.DeltaArgs()
     a.o, a.d_o, a.delta = o.data_ptr(), do.data_ptr(), delta.data_ptr()
     a.B, a.Hq, a.D, a.Sq = B, Hq, D, Sq
@@ -193,6 +197,11 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     if dkdv_direct:
         for t in list(dk_accs) + list(dv_accs):
             _req(t, "dK / dV")
+    if q.numel() == 0:          # no query rows: nothing to add; results that this call was to write are zero
+        if dkdv_direct and do_dkdv:
+            for t in list(dk_accs) + list(dv_accs):
+                t.zero_()
+        return
     a = _lib.BwdArgs()
     a.q, a.d_o, a.lse, a.dq = q.data_ptr(), do.data_ptr(), lse.data_ptr(), dq_acc.data_ptr()
     a.delta = None if library_scratch else delta.data_ptr()

@@ -973,3 +973,25 @@ def test_dkdv_keys_256_refused_where_it_does_not_exist(ltr):
         ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dkdv_keys=64)
     with pytest.raises(RuntimeError):
         ltr.attn_bwd_accumulate(q, do, lse, delta, [k], [v], [0], dq, [dk], [dv], dq_rows=512)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_no_query_rows(ltr, dtype):
+    """A rank whose q chunk is empty (the reference's matmuls return an empty result there, ring_attention.py:66-104):
+    empty O and LSE, zero gradients for K and V, no kernel launch and no error."""
+    g = torch.Generator().manual_seed(5)
+    q = torch.zeros(2, 0, 4, 64, dtype=dtype).cuda().requires_grad_(True)
+    k, v = _dev(_randn((2, 48, 2, 64), g, dtype), _randn((2, 48, 2, 64), g, dtype))
+    k.requires_grad_(True)
+    v.requires_grad_(True)
+    o, lse = ltr.block_attention(q, [k], [v], [0], 0, None, True)
+    assert tuple(o.shape) == (2, 0, 4, 64) and tuple(lse.shape) == (2, 4, 0) and o.dtype == dtype
+    o.sum().backward()
+    torch.cuda.synchronize()
+    assert tuple(q.grad.shape) == (2, 0, 4, 64)
+    assert k.grad is not None and v.grad is not None
+    assert float(k.grad.float().abs().max()) == 0.0 and float(v.grad.float().abs().max()) == 0.0
+    # the low-level calls as well
+    o2, lse2 = ltr.attn_fwd(q.detach(), [k.detach()], [v.detach()], [0])
+    assert o2.numel() == 0 and lse2.numel() == 0
+    assert ltr.attn_delta(o2, o2).numel() == 0
