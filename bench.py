@@ -352,7 +352,7 @@ def _run_attention(la, torch, cfg, steps, warmup, data="randn", min_warm_s=0.0, 
         # template arguments: head dim, 32-key halves per wave (2 = the 256-key blocks the library picks for long head-dim-64 streams)
         dom, dom_ms, dom_flops = "bwd_dkdv_kernel<%d, %d>" % (D, 2 if (D == 64 and not causal and S >= 4096) else 1), dkdv_ms, 2.0 * f_share
     else:
-        dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d>" % D, fwd_ms, f_share
+        dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d, 1>" % D, fwd_ms, f_share
     return {"dt": dt, "f_total": f_total, "kernels": kernels, "launches": launches, "steps": steps, "warmup": n_warm,
             "dominant": (dom, dom_flops / (dom_ms * 1e-3) / 1e12)}
 

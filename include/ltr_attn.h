@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 6
+#define LTR_ABI_VERSION 7
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -61,6 +61,9 @@ extern "C" {
                                    do not depend on the hint beyond the order of fp32 additions inside a block */
 #define LTR_DQ_ROWS_256 2048u /* backward, tuning hint: the dQ kernel's blocks own 256 query rows (the default choice is the library's) */
 #define LTR_DQ_ROWS_512 4096u /* backward, tuning hint: they own 512 rows (bf16, head dim 64 only: LTR_EUNSUP otherwise); same results */
+#define LTR_FWD_ROWS_256 8192u  /* forward, tuning hint: the kernel's blocks own 256 query rows (the default choice is the library's) */
+#define LTR_FWD_ROWS_512 16384u /* forward, tuning hint: they own 512 rows (bf16, head dim 64 only: LTR_EUNSUP otherwise); results differ
+                                   only through the tile size (64 instead of 128 keys: the order of fp32 additions) */
 
 /* error codes */
 #define LTR_OK 0
@@ -107,7 +110,7 @@ typedef struct ltr_attn_fwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;          /* 1/sqrt(D) at every reference call site (ring_attention.py:20) */
-    uint32_t flags;
+    uint32_t flags;       /* LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q | LTR_FWD_ROWS_256 | LTR_FWD_ROWS_512 */
     int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v */
     int32_t o_dtype;      /* LTR_BF16 or LTR_F32 */
     int32_t n_chunks;     /* 1..LTR_MAX_CHUNKS */

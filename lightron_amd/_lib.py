@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # LTR_ATTN_LIB names another build of the same library (same ABI version), e.g. to compare two builds in one session
 LIB_PATH = os.environ.get("LTR_ATTN_LIB") or os.path.join(HERE, "csrc", "libltr_attn.so")
 
-LTR_ABI_VERSION = 6
+LTR_ABI_VERSION = 7
 LTR_MAX_CHUNKS = 32
 LTR_NOALLOC_MAX_ROWS = 1 << 20
 LTR_BF16, LTR_F32 = 0, 1
@@ -16,6 +16,7 @@ LTR_CAUSAL, LTR_MERGE, LTR_NO_DQ, LTR_NO_DKDV, LTR_DQ_BF16, LTR_DELTA_FROM_O, LT
 LTR_ROPE_Q, LTR_ROPE_DQ = 128, 256
 LTR_DKDV_KEYS_128, LTR_DKDV_KEYS_256 = 512, 1024
 LTR_DQ_ROWS_256, LTR_DQ_ROWS_512 = 2048, 4096
+LTR_FWD_ROWS_256, LTR_FWD_ROWS_512 = 8192, 16384
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
            "ltr_device_info", "ltr_probe_mfma", "ltr_probe_atomic_tile_add", "ltr_abi_version", "ltr_strerror")

@@ -74,11 +74,12 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
              q_pos0=0, q_split: Optional[int] = None, causal: bool = False, scale: Optional[float] = None,
              out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None, merge: bool = False,
              out_dtype: Optional[torch.dtype] = None, q_rope: Optional[torch.Tensor] = None,
-             q_rot_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+             q_rot_out: Optional[torch.Tensor] = None, fwd_rows: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """One Q chunk against a table of KV chunks -> (O [B,Sq,Hq,D], LSE [B,Hq,Sq] fp32).
     With merge=True, `out`/`lse` hold an earlier partial result which is merged in place.
     q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table whose row p belongs to global position p: q is un-rotated and the
-    kernel's prologue applies RoPE to it (LTR_ROPE_Q; bf16 only); q_rot_out (bf16, like q) receives the rotated q."""
+    kernel's prologue applies RoPE to it (LTR_ROPE_Q; bf16 only); q_rot_out (bf16, like q) receives the rotated q.
+    fwd_rows: None (the library chooses), 256 or 512 query rows per block (512: bf16 with head dim 64 only)."""
     lib = _lib.load()
     _req(q, "q")
     B, Sq, Hq, D = q.shape
@@ -110,10 +111,14 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
     a.io_dtype, a.o_dtype = _DT[q.dtype], _DT[out.dtype]
     rope_flag = 0
+    if fwd_rows is not None:
+        if fwd_rows not in (256, 512):
+            raise RuntimeError("fwd_rows must be None, 256 or 512")
+        rope_flag |= _lib.LTR_FWD_ROWS_256 if fwd_rows == 256 else _lib.LTR_FWD_ROWS_512
     if q_rope is not None:
         _rope_table_check(q_rope, D, q.device)
         a.rope_freqs, a.rope_pos0, a.rope_len = q_rope.data_ptr(), 0, q_rope.shape[0]
-        rope_flag = _lib.LTR_ROPE_Q
+        rope_flag |= _lib.LTR_ROPE_Q
         if q_rot_out is not None:
             _req(q_rot_out, "q_rot_out")
             if q_rot_out.dtype != torch.bfloat16 or q_rot_out.shape != q.shape:

@@ -2,8 +2,8 @@
 // KV chunks resident in HBM, recompute backward, behind the C ABI of include/ltr_attn.h.
 //
 // Kernel map
-//   fwd_bf16_kernel<D>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a block of
-//                        8 waves owns 256 query rows, a wave 32 of them, so a lane owns ONE query:
+//   fwd_bf16_kernel<D, RB>   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16; a block of
+//                        8 waves owns 256 * RB query rows, a wave 32 * RB of them, so a lane owns ONE query per row block:
 //                        the row sums are in-lane reductions (no running max: the reference of the
 //                        exponent moves only when a row sum leaves its safe range), and P^T leaves the
 //                        first GEMM already in the B-operand layout of the second.  64-key K
@@ -11,6 +11,8 @@
 //                        unpadded, XOR-swizzled, double-buffered tiles, one barrier per tile;
 //                        the V^T operand is read with ds_read_b64_tr_b16.  The (O, LSE) merge
 //                        with an earlier partial result is part of the epilogue.
+//                        fwd_bf16_kernel<64, 2>: two 32-row blocks per wave (512 rows per block, 64-key tiles): every K / V
+//                        operand read from LDS feeds two MFMAs (chosen by the host, or forced with LTR_FWD_ROWS_512).
 //   fwd_f32_kernel<D>    fp32 I/O and arithmetic (no MFMA), for the 1e-4 parity case.
 //   delta_kernel         DELTA = rowsum(dO * O).
 //   bwd_dkdv_kernel<D, KW>  a block of 8 waves owns 128 * KW keys of one kv head and loops over the
@@ -455,17 +457,60 @@ __device__ __forceinline__ void wave_tile_rowmajor(unsigned char *stage, int lan
     }
 }
 
+// lds_gemm_chain / lds_tr_gemm for a wave that owns KW 32-key halves (dK/dV kernel) or KW 32-row blocks (forward): every operand
+// read from LDS feeds one MFMA per half (b[k], r[k] / acc[k] belong to half k); hook(step) follows the MFMAs of operand `step`.
+template <int D, int KW, class Hook = NoHook>
+__device__ __forceinline__ void lds_gemm_chain_kw(const __bf16 *row, int sw, const bf16x8 (&b)[KW][D / 16], f32x16 (&r)[KW],
+                                                  Hook hook = Hook()) {
+    constexpr int NK = D / 16, PF = 2;
+    bf16x8 x[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF; i++) x[i] = *(const bf16x8 *)(row + (((2 * i) ^ sw) << 3));
+#pragma unroll
+    for (int kb = 0; kb < NK; kb++) {
+        if (kb + PF < NK) x[(kb + PF) % (PF + 1)] = *(const bf16x8 *)(row + (((2 * (kb + PF)) ^ sw) << 3));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < KW; k++) r[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[kb % (PF + 1)], b[k][kb], r[k], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        hook(kb);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+template <int D, int NKB, int KW, class Hook = NoHook>
+__device__ __forceinline__ void lds_tr_gemm_kw(const __bf16 *T, int row0, int lane, const bf16x8 (&b)[KW][NKB],
+                                               f32x16 (&acc)[KW][D / 32], Hook hook = Hook()) {
+    constexpr int ND = D / 32, N = NKB * ND, PF = 3;
+    bf16x8 a[PF + 1];
+#pragma unroll
+    for (int i = 0; i < PF && i < N; i++) a[i] = lds_operand_tr_swz<D>(T, row0 + (i / ND) * 16, (i % ND) * 32, lane);
+#pragma unroll
+    for (int step = 0; step < N; step++) {
+        if (step + PF < N)
+            a[(step + PF) % (PF + 1)] = lds_operand_tr_swz<D>(T, row0 + ((step + PF) / ND) * 16, ((step + PF) % ND) * 32, lane);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < KW; k++)
+            acc[k][step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[k][step / ND], acc[k][step % ND], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        hook(step);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // keys per K / V tile of the forward and dQ kernels
-template <int D>
+template <int D, int RB = 1>
 struct FwdTile {
-    static constexpr int BN = D == 64 ? 128 : 64;
+    static constexpr int BN = (D == 64 && RB == 1) ? 128 : 64;   // two row blocks per wave: S^T of 128 keys would be 128 registers
 };
 
 // ------------------------------------------------------------------------------ forward, bf16
-template <int D>
+// RB = 32-row blocks per wave.  With two (head dim 64) every K / V operand read from LDS feeds two MFMAs and a tile of
+// 64 keys serves 512 query rows: half the LDS reads and half the tile transfers per MFMA.
+template <int D, int RB>
 __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
-    constexpr int NW = 8, BM = 32 * NW;   // 8 waves (two per SIMD) share every K / V tile
-    constexpr int BN = FwdTile<D>::BN, NB = BN / 32;   // keys per tile: a tile moves 32 KB whatever the head dim
+    constexpr int NW = 8, BM = 32 * RB * NW;   // 8 waves (two per SIMD) share every K / V tile
+    constexpr int BN = FwdTile<D, RB>::BN, NB = BN / 32;   // keys per tile: 32 KB (16 KB with two row blocks per wave)
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide 16-byte-per-lane LDS-direct load (1 KB)
     constexpr int NI = BN / (RPI * NW);       // such loads per wave, per tensor and per tile
@@ -508,36 +553,42 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     const int lane = lane_of_part, l32 = lane & 31, hh = lane >> 5;
 
     const int row0 = qt * BM;
-    const int my_row = row0 + w * 32 + l32;
-    const bool row_ok = my_row < p.Sq;
-    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int my_row[RB], my_pos[RB];   // row block rb of wave w: rows row0 + 32 * (RB * w + rb) ..
+    bool row_ok[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        my_row[rb] = row0 + (w * RB + rb) * 32 + l32;
+        row_ok[rb] = my_row[rb] < p.Sq;
+        my_pos[rb] = q_position(my_row[rb], p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    }
     int blk_lo, blk_hi, w_lo, w_hi;
     q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
     {
-        int wr0 = row0 + w * 32, wr1 = min(wr0 + 32, p.Sq) - 1;
+        int wr0 = row0 + w * 32 * RB, wr1 = min(wr0 + 32 * RB, p.Sq) - 1;
         if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
         else { w_lo = 0x7fffffff; w_hi = -0x7fffffff; }  // wave has no valid row
     }
 
     // Q operand (B of S^T = K Q^T): lane (query l32, half hh) holds d = 16*kb + 8*hh .. +7
-    bf16x8 qreg[D / 16];
-    {
-        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + (long long)my_row * p.qs[1] + h * p.qs[2];
+    bf16x8 qreg[RB][D / 16];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + (long long)my_row[rb] * p.qs[1] + h * p.qs[2];
 #pragma unroll
         for (int kb = 0; kb < D / 16; kb++) {
             uint4 x = make_uint4(0, 0, 0, 0);
-            if (row_ok) x = *(const uint4 *)(qp + kb * 16 + 8 * hh);
-            qreg[kb] = as_bf16x8(x);
+            if (row_ok[rb]) x = *(const uint4 *)(qp + kb * 16 + 8 * hh);
+            qreg[rb][kb] = as_bf16x8(x);
         }
         // fused RoPE prologue: q arrives un-rotated and is rotated here, in the registers that hold it as the MFMA operand,
         // by the angles of the row's global position; the rotated row can be stored for the backward
-        if ((p.flags & LTR_ROPE_Q) && row_ok) {
-            const float *fr = p.rope + (long long)(my_pos - p.rope_pos0) * D + 8 * hh;
-            __bf16 *qr = p.q_rot ? (__bf16 *)p.q_rot + b * p.qrs[0] + (long long)my_row * p.qrs[1] + h * p.qrs[2] + 8 * hh : nullptr;
+        if ((p.flags & LTR_ROPE_Q) && row_ok[rb]) {
+            const float *fr = p.rope + (long long)(my_pos[rb] - p.rope_pos0) * D + 8 * hh;
+            __bf16 *qr = p.q_rot ? (__bf16 *)p.q_rot + b * p.qrs[0] + (long long)my_row[rb] * p.qrs[1] + h * p.qrs[2] + 8 * hh : nullptr;
 #pragma unroll
             for (int kb = 0; kb < D / 16; kb++) {
-                qreg[kb] = rope_rotate8(qreg[kb], *(const f32x4 *)(fr + 16 * kb), *(const f32x4 *)(fr + 16 * kb + 4));
-                if (qr) *(bf16x8 *)(qr + 16 * kb) = qreg[kb];
+                qreg[rb][kb] = rope_rotate8(qreg[rb][kb], *(const f32x4 *)(fr + 16 * kb), *(const f32x4 *)(fr + 16 * kb + 4));
+                if (qr) *(bf16x8 *)(qr + 16 * kb) = qreg[rb][kb];
             }
         }
     }
@@ -545,17 +596,23 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     f32x16 zero16;
 #pragma unroll
     for (int r = 0; r < 16; r++) zero16[r] = 0.f;
-    f32x16 oacc[D / 32];
+    f32x16 oacc[RB][D / 32];
 #pragma unroll
-    for (int i = 0; i < D / 32; i++) oacc[i] = zero16;
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int i = 0; i < D / 32; i++) oacc[rb][i] = zero16;
     // Online softmax state of this lane's query row.  mc is the reference point of the exponent (exp2 domain:
     // m * scale * log2(e)).  It does not follow the running max: P = exp2(s*c2 - mc) keeps its relative precision
     // whatever mc is, l and O accumulate in fp32 and LSE = mc*ln2 + log(l) is unaffected, so mc only has to keep
     // the row sum inside [TINY, BIG] where neither overflow nor flushed small terms matter.  That is checked on
     // the row sum of each tile (two compares), and the row max is only computed on the rare tile that fails the
     // check: the common tile has no max reduction and no rescale of the O accumulator.
-    float mc = 0.f;
-    float l_run = 0.f;        // this lane's partial row sum (its half of the keys of every tile)
+    float mc[RB], l_run[RB];  // l_run: this lane's partial row sum (its half of the keys of every tile)
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        mc[rb] = 0.f;
+        l_run[rb] = 0.f;
+    }
     const float c2 = p.scale * LTR_LOG2E;
     constexpr float BIG = 1.152921504606846976e18f, TINY = 8.673617379884035472e-19f;   // 2^60, 2^-60
 
@@ -637,90 +694,118 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         // S^T of the two 32-key blocks of the tile.  The wave raises its priority while it issues MFMAs: the
         // other wave of the SIMD then fills the gaps with its softmax arithmetic instead of delaying them.
         __builtin_amdgcn_s_setprio(1);
-        f32x16 s[NB];
+        f32x16 s[NB][RB];
+        if constexpr (RB == 1) {
 #pragma unroll
-        for (int nb = 0; nb < NB; nb += 2) {
-            s[nb] = zero16;
-            s[nb + 1] = zero16;
-            lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, lds_swz<D>(nb * 32 + l32) ^ hh, Ks + (nb * 32 + 32 + l32) * D,
-                             lds_swz<D>(nb * 32 + 32 + l32) ^ hh, qreg, qreg, s[nb], s[nb + 1]);
+            for (int nb = 0; nb < NB; nb += 2) {
+                s[nb][0] = zero16;
+                s[nb + 1][0] = zero16;
+                lds_gemm_pair<D>(Ks + (nb * 32 + l32) * D, lds_swz<D>(nb * 32 + l32) ^ hh, Ks + (nb * 32 + 32 + l32) * D,
+                                 lds_swz<D>(nb * 32 + 32 + l32) ^ hh, qreg[0], qreg[0], s[nb][0], s[nb + 1][0]);
+            }
+        } else {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++) s[nb][rb] = zero16;
+                lds_gemm_chain_kw<D, RB>(Ks + (nb * 32 + l32) * D, lds_swz<D>(nb * 32 + l32) ^ hh, qreg, s[nb]);
+            }
         }
         __builtin_amdgcn_s_setprio(0);
         // mask fix-up (tail of the chunk, diagonal tiles): wave-uniform branch touching S only
         const bool need_mask = (key0 + BN > sk) || (causal && (pos0 + key0 + BN - 1 > w_lo));
         if (need_mask) {
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++)
+            for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
-                    const bool vis = key < sk && (!causal || pos0 + key <= my_pos);
-                    s[nb][r] = vis ? s[nb][r] : -INFINITY;
-                }
+                for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int key = key0 + nb * 32 + 8 * (r / 4) + 4 * hh + (r % 4);
+                        const bool vis = key < sk && (!causal || pos0 + key <= my_pos[rb]);
+                        s[nb][rb][r] = vis ? s[nb][rb][r] : -INFINITY;
+                    }
         }
         // t = s*c2 - reference (exp2 domain), P = exp2(t) rounded to bf16, row sum of the rounded P (what PV uses)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
+        for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[nb][r] = s[nb][r] * c2 - mc;
-        PackedTile pt[NB];
+            for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[nb][rb][r] = s[nb][rb][r] * c2 - mc[rb];
+        PackedTile pt[RB][NB];
         bf16x2 ones;
         ones[0] = (__bf16)1.0f;
         ones[1] = (__bf16)1.0f;
-        float l_tile = 0.f;
-        auto exponentials = [&]() {
-            l_tile = 0.f;
+        float l_tile[RB];
+        auto exponentials = [&](int rb) {
+            l_tile[rb] = 0.f;
 #pragma unroll
             for (int nb = 0; nb < NB; nb++)
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     bf16x2 pr;
-                    pr[0] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j]);
-                    pr[1] = (__bf16)__builtin_amdgcn_exp2f(s[nb][2 * j + 1]);
-                    l_tile = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_tile, false);
-                    pt[nb].u[j] = __builtin_bit_cast(unsigned, pr);
+                    pr[0] = (__bf16)__builtin_amdgcn_exp2f(s[nb][rb][2 * j]);
+                    pr[1] = (__bf16)__builtin_amdgcn_exp2f(s[nb][rb][2 * j + 1]);
+                    l_tile[rb] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, l_tile[rb], false);
+                    pt[rb][nb].u[j] = __builtin_bit_cast(unsigned, pr);
                 }
         };
-        exponentials();
-        // in range: the tile's sum did not overflow and the row has a healthy sum by now (a lane sees half of the
-        // row's keys, so its partial sum can lag behind the row's: that only costs a visit of the branch below)
-        const bool out_of_range = !(l_tile < BIG) || !(l_run + l_tile >= TINY);
-        if (__builtin_amdgcn_ballot_w64(out_of_range) != 0) {
-            float mx = -INFINITY;
+        bool out_of_range = false;
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[nb][r]);
-            mx = xhalf_max(mx);                       // row max of t over the tile (-inf: no visible key)
-            const float l_row = xhalf_sum(l_run), lt_row = xhalf_sum(l_tile);   // whole-row sums: both halves agree
-            const bool row_bad = !(lt_row < BIG) || !(l_row + lt_row >= TINY);
-            // New reference for a row that is out of range: the larger of the tile's max and the magnitude of the
-            // history (log2 of its sum), so that neither overflows after the move; with a history never below -126, so
-            // that the factor applied to it stays finite.  Rows that are in range, and rows that have seen no key at
-            // all, keep theirs.
-            const float hist = l_row > 0.f ? __log2f(l_row) : -INFINITY;
-            const float target = fmaxf(mx, hist);
-            const float shift = (row_bad && target > -INFINITY) ? (l_row > 0.f ? fmaxf(target, -126.f) : target) : 0.f;
-            const float alpha = l_row > 0.f ? __builtin_amdgcn_exp2f(-shift) : 1.f;
-            l_run *= alpha;
-#pragma unroll
-            for (int i = 0; i < D / 32; i++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) s[nb][r] -= shift;
-            mc += shift;
-            exponentials();
+        for (int rb = 0; rb < RB; rb++) {
+            exponentials(rb);
+            // in range: the tile's sum did not overflow and the row has a healthy sum by now (a lane sees half of the
+            // row's keys, so its partial sum can lag behind the row's: that only costs a visit of the branch below)
+            out_of_range = out_of_range || !(l_tile[rb] < BIG) || !(l_run[rb] + l_tile[rb] >= TINY);
         }
-        l_run += l_tile;
+        if (__builtin_amdgcn_ballot_w64(out_of_range) != 0) {
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[nb][rb][r]);
+                mx = xhalf_max(mx);                       // row max of t over the tile (-inf: no visible key)
+                const float l_row = xhalf_sum(l_run[rb]), lt_row = xhalf_sum(l_tile[rb]);   // whole-row sums: both halves agree
+                const bool row_bad = !(lt_row < BIG) || !(l_row + lt_row >= TINY);
+                // New reference for a row that is out of range: the larger of the tile's max and the magnitude of the
+                // history (log2 of its sum), so that neither overflows after the move; with a history never below -126, so
+                // that the factor applied to it stays finite.  Rows that are in range, and rows that have seen no key at
+                // all, keep theirs.
+                const float hist = l_row > 0.f ? __log2f(l_row) : -INFINITY;
+                const float target = fmaxf(mx, hist);
+                const float shift = (row_bad && target > -INFINITY) ? (l_row > 0.f ? fmaxf(target, -126.f) : target) : 0.f;
+                const float alpha = l_row > 0.f ? __builtin_amdgcn_exp2f(-shift) : 1.f;
+                l_run[rb] *= alpha;
+#pragma unroll
+                for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) oacc[rb][i][r] *= alpha;
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s[nb][rb][r] -= shift;
+                mc[rb] += shift;
+                exponentials(rb);
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) l_run[rb] += l_tile[rb];
         __builtin_amdgcn_s_setprio(1);
-        {
+        if constexpr (RB == 1) {
             bf16x8 pb[2 * NB];
 #pragma unroll
-            for (int kb = 0; kb < 2 * NB; kb++) pb[kb] = operand_of(pt[kb >> 1], kb & 1);
-            lds_tr_gemm<D, 2 * NB>(Vs, 0, lane, pb, oacc);   // 16 keys per MFMA
+            for (int kb = 0; kb < 2 * NB; kb++) pb[kb] = operand_of(pt[0][kb >> 1], kb & 1);
+            lds_tr_gemm<D, 2 * NB>(Vs, 0, lane, pb, oacc[0]);   // 16 keys per MFMA
+        } else {
+            bf16x8 pb[RB][2 * NB];
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int kb = 0; kb < 2 * NB; kb++) pb[rb][kb] = operand_of(pt[rb][kb >> 1], kb & 1);
+            lds_tr_gemm_kw<D, 2 * NB, RB>(Vs, 0, lane, pb, oacc);   // 16 keys per MFMA, one V operand read for both row blocks
         }
         __builtin_amdgcn_s_setprio(0);
         }
@@ -733,13 +818,16 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         tile_step(std::integral_constant<int, 1>{});
     }
 
-    // epilogue: normalise, optional merge with the partial result already in (o, lse)
-    const float l_tot = xhalf_sum(l_run);
-    float lse_new = (l_tot > 0.f) ? mc * LTR_LN2 + logf(l_tot) : -INFINITY;
+    // epilogue: normalise, optional merge with the partial result already in (o, lse); one row block after the other
+    // through the same staging area
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+    const float l_tot = xhalf_sum(l_run[rb]);
+    float lse_new = (l_tot > 0.f) ? mc[rb] * LTR_LN2 + logf(l_tot) : -INFINITY;
     float w_cur = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     float w_old = 0.f;
-    float *lse_p = p.lse + ((long long)b * p.Hq + h) * p.Sq + my_row;
-    if ((p.flags & LTR_MERGE) && row_ok) {
+    float *lse_p = p.lse + ((long long)b * p.Hq + h) * p.Sq + my_row[rb];
+    if ((p.flags & LTR_MERGE) && row_ok[rb]) {
         const float lse_old = *lse_p;
         const float mxl = fmaxf(lse_old, lse_new);
         if (mxl == -INFINITY) {
@@ -752,13 +840,13 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             lse_new = mxl + logf(tot);
         }
     }
-    if (row_ok && hh == 0) *lse_p = lse_new;
+    if (row_ok[rb] && hh == 0) *lse_p = lse_new;
     // O through the wave's LDS staging area (the tiles are no longer read: the last barrier is behind us)
     unsigned char *stage = smem + w * WaveStage<D>::BYTES;
     float *row_w_old = (float *)(stage + 32 * WaveStage<D>::ROW_BYTES);
     if (hh == 0) row_w_old[l32] = w_old;
     constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;      // see wave_tile_rowmajor
-    const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + w * 32);
+    const int Sq_u = uniform32(p.Sq), wave_row0 = uniform32(row0 + (w * RB + rb) * 32);
     const bool merge = uniform32(p.flags & LTR_MERGE) != 0, o_f32 = uniform32(p.o_f32) != 0;
     const long long os1 = uniform64(p.os[1]);
     const long long off0 = uniform64(b * p.os[0] + h * p.os[2]) + (wave_row0 + lane / LPR) * os1 + 4 * (lane % LPR);
@@ -781,7 +869,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     int it = 0;
     if (o_f32) {
         float *op = (float *)p.o + off0;
-        wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
+        wave_tile_rowmajor<D>(stage, lane, oacc[rb], w_cur, [&](int row, int, f32x4 val) {
             if (wave_row0 + row < Sq_u) {
                 if (merge) {
                     const float wo = row_w_old[row];
@@ -795,7 +883,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
         });
     } else {
         __bf16 *op = (__bf16 *)p.o + off0;
-        wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
+        wave_tile_rowmajor<D>(stage, lane, oacc[rb], w_cur, [&](int row, int, f32x4 val) {
             if (wave_row0 + row < Sq_u) {
                 if (merge) {
                     const float wo = row_w_old[row];
@@ -811,6 +899,7 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
             it++;
         });
     }
+    }   // row block
     }   // part
 }
 
@@ -1012,47 +1101,6 @@ __device__ __forceinline__ unsigned bwd_p_pair(const f32x16 &sm, int j, float c2
 __device__ __forceinline__ unsigned bwd_ds_pair(unsigned pu, const f32x16 &dpm, int j) {
     const float p0 = __uint_as_float(pu << 16), p1 = __uint_as_float(pu & 0xffff0000u);
     return pack2_bf16(p0 * dpm[2 * j], p1 * dpm[2 * j + 1]);
-}
-
-// lds_gemm_chain / lds_tr_gemm for a wave that owns KW 32-key halves: every operand read from LDS feeds one MFMA per half
-// (b[k], r[k] / acc[k] belong to half k); hook(step) follows the MFMAs of operand `step`.
-template <int D, int KW, class Hook = NoHook>
-__device__ __forceinline__ void lds_gemm_chain_kw(const __bf16 *row, int sw, const bf16x8 (&b)[KW][D / 16], f32x16 (&r)[KW],
-                                                  Hook hook = Hook()) {
-    constexpr int NK = D / 16, PF = 2;
-    bf16x8 x[PF + 1];
-#pragma unroll
-    for (int i = 0; i < PF; i++) x[i] = *(const bf16x8 *)(row + (((2 * i) ^ sw) << 3));
-#pragma unroll
-    for (int kb = 0; kb < NK; kb++) {
-        if (kb + PF < NK) x[(kb + PF) % (PF + 1)] = *(const bf16x8 *)(row + (((2 * (kb + PF)) ^ sw) << 3));
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int k = 0; k < KW; k++) r[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[kb % (PF + 1)], b[k][kb], r[k], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        hook(kb);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-}
-template <int D, int NKB, int KW, class Hook = NoHook>
-__device__ __forceinline__ void lds_tr_gemm_kw(const __bf16 *T, int row0, int lane, const bf16x8 (&b)[KW][NKB],
-                                               f32x16 (&acc)[KW][D / 32], Hook hook = Hook()) {
-    constexpr int ND = D / 32, N = NKB * ND, PF = 3;
-    bf16x8 a[PF + 1];
-#pragma unroll
-    for (int i = 0; i < PF && i < N; i++) a[i] = lds_operand_tr_swz<D>(T, row0 + (i / ND) * 16, (i % ND) * 32, lane);
-#pragma unroll
-    for (int step = 0; step < N; step++) {
-        if (step + PF < N)
-            a[(step + PF) % (PF + 1)] = lds_operand_tr_swz<D>(T, row0 + ((step + PF) / ND) * 16, ((step + PF) % ND) * 32, lane);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int k = 0; k < KW; k++)
-            acc[k][step % ND] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step % (PF + 1)], b[k][step / ND], acc[k][step % ND], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        hook(step);
-        __builtin_amdgcn_sched_barrier(0);
-    }
 }
 
 template <int D, int KW>
@@ -2089,9 +2137,9 @@ int check_device() {   // gfx950 only
 }
 
 // kernels that need more than 64 KB of dynamic LDS must opt in once per device
-template <int D>
+template <int D, int RB = 1>
 constexpr int fwd_lds_bytes() {   // the K / V tile buffers, reused by the epilogue's staging areas (one per wave)
-    return 2 * 2 * FwdTile<D>::BN * D * 2 > 8 * WaveStage<D>::BYTES ? 2 * 2 * FwdTile<D>::BN * D * 2 : 8 * WaveStage<D>::BYTES;
+    return 2 * 2 * FwdTile<D, RB>::BN * D * 2 > 8 * WaveStage<D>::BYTES ? 2 * 2 * FwdTile<D, RB>::BN * D * 2 : 8 * WaveStage<D>::BYTES;
 }
 template <int D>
 constexpr int dq_lds_bytes() { return fwd_lds_bytes<D>(); }   // same tile buffers and staging areas as the forward
@@ -2106,10 +2154,12 @@ int enable_large_lds() {
                                   BwdLds<64, 1>::TOTAL) == hipSuccess &&
               hipFuncSetAttribute((const void *)bwd_dkdv_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   BwdLds<64, 2>::TOTAL) == hipSuccess &&
-              hipFuncSetAttribute((const void *)fwd_bf16_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+              hipFuncSetAttribute((const void *)fwd_bf16_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   fwd_lds_bytes<128>()) == hipSuccess &&
-              hipFuncSetAttribute((const void *)fwd_bf16_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+              hipFuncSetAttribute((const void *)fwd_bf16_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   fwd_lds_bytes<64>()) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_bf16_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  fwd_lds_bytes<64, 2>()) == hipSuccess &&
               hipFuncSetAttribute((const void *)bwd_dq_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<128>()) == hipSuccess &&
               hipFuncSetAttribute((const void *)bwd_dq_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -2236,7 +2286,8 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     if (!a || !a->q || !a->o || !a->lse) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q)) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q | LTR_FWD_ROWS_256 | LTR_FWD_ROWS_512)) return LTR_EINVAL;
+    if ((a->flags & LTR_FWD_ROWS_256) && (a->flags & LTR_FWD_ROWS_512)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     if (a->o_dtype != LTR_BF16 && a->o_dtype != LTR_F32) return LTR_EUNSUP;
@@ -2297,20 +2348,35 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     p.q_pos0[1] = (int)a->q_pos0[1];
     p.q_split = (int)a->q_split;
     p.scale = a->scale;
-    p.flags = a->flags;
+    p.flags = a->flags & (LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q);
     p.o_f32 = a->o_dtype == LTR_F32;
     p.n_chunks = a->n_chunks;
     hipStream_t st = (hipStream_t)stream;
+    if ((a->flags & LTR_FWD_ROWS_512) && (a->D != 64 || a->io_dtype != LTR_BF16)) return LTR_EUNSUP;
     if (a->io_dtype == LTR_BF16) {
-        p.n_qtiles = (p.Sq + 255) / 256;
-        if ((long long)p.n_qtiles * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
+        if ((long long)((p.Sq + 255) / 256) * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
+        const bool causal_ = (p.flags & LTR_CAUSAL) != 0;
+        // query rows per block: 512 (two 32-row blocks per wave, 64-key tiles) pays at head dim 64 under the conditions of
+        // the dQ kernel's 512-row blocks (see bwd_launch)
+        bool wide = (a->flags & LTR_FWD_ROWS_512) != 0;
+        if (!wide && !(a->flags & LTR_FWD_ROWS_256) && a->D == 64) {
+            const int tiles512 = (p.Sq + 511) / 512;
+            const int slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_ && q_tiles_uneven(p.Sq, 512, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
+            const long long blocks512 = (long long)slots512 * p.B * p.Hq, blocks256 = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
+            const int cus = device_cus();
+            wide = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus)
+                           : (cu_fill(blocks512, cus) * 1.07 >= cu_fill(blocks256, cus));
+        }
+        const int rows = wide ? 512 : 256;
+        p.n_qtiles = (p.Sq + rows - 1) / rows;
         p.n_slots = q_tile_slots(p.n_qtiles, (long long)p.B * p.Hq,
-                                 (p.flags & LTR_CAUSAL) && q_tiles_uneven(p.Sq, 256, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
+                                 causal_ && q_tiles_uneven(p.Sq, rows, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
         const long long nblk = (long long)p.n_slots * p.B * p.Hq;
         rc = enable_large_lds();
         if (rc) return rc;
-        if (a->D == 128) hipLaunchKernelGGL(fwd_bf16_kernel<128>, dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<128>(), st, p);
-        else hipLaunchKernelGGL(fwd_bf16_kernel<64>, dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<64>(), st, p);
+        if (a->D == 128) hipLaunchKernelGGL((fwd_bf16_kernel<128, 1>), dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<128>(), st, p);
+        else if (wide) hipLaunchKernelGGL((fwd_bf16_kernel<64, 2>), dim3((unsigned)nblk), dim3(512), (fwd_lds_bytes<64, 2>()), st, p);
+        else hipLaunchKernelGGL((fwd_bf16_kernel<64, 1>), dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<64>(), st, p);
     } else {
         p.n_qtiles = (p.Sq + 63) / 64;
         p.n_slots = p.n_qtiles;

@@ -995,3 +995,87 @@ def test_no_query_rows(ltr, dtype):
     o2, lse2 = ltr.attn_fwd(q.detach(), [k.detach()], [v.detach()], [0])
     assert o2.numel() == 0 and lse2.numel() == 0
     assert ltr.attn_delta(o2, o2).numel() == 0
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_fwd_block_size_hints_d64(ltr, seed):
+    """Head dim 64: the forward kernel with 256 and with 512 query rows per block (LTR_FWD_ROWS_256 / _512, the latter two
+    32-row blocks per wave and 64-key tiles), forced through the hint flags: ragged rows and chunks, several chunks, GQA,
+    causal with a two-segment query (so that the paired and the unpaired hand-out of q tiles both occur), bf16 and fp32
+    output, one launch or a stepwise merge, optionally with the fused RoPE prologue.  Both against the dense oracle and
+    against each other to rounding; the rotated q must have the same bits."""
+    import random
+    rnd = random.Random(9000 + seed)
+    g = torch.Generator().manual_seed(9500 + seed)
+    D = 64
+    Hkv = rnd.choice([1, 2])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    B = rnd.choice([1, 2])
+    Sq = rnd.choice([31, 64, 300, 512, 513, 700, 1024, 1300])
+    n_ch = rnd.randint(1, 3)
+    sks = [rnd.choice([1, 33, 64, 100, 128, 191, 257, 330, 600]) for _ in range(n_ch)]
+    causal = rnd.random() < 0.6
+    out_dtype = rnd.choice([torch.bfloat16, torch.float32])
+    stepwise = n_ch > 1 and rnd.random() < 0.5
+    rope = rnd.random() < 0.4
+    starts, p = [], rnd.randint(0, 30)
+    for sk in sks:
+        starts.append(p)
+        p += sk + rnd.randint(0, 20)
+    q_split = rnd.choice([None, rnd.randint(1, Sq - 1)])
+    if q_split is None:
+        qp = rnd.randint(0, p + 400)
+        q_pos, q_pos0 = torch.arange(qp, qp + Sq), qp
+    else:
+        a0, a1 = rnd.randint(0, p), rnd.randint(0, p + 400)
+        q_pos = torch.cat([torch.arange(a0, a0 + q_split), torch.arange(a1, a1 + Sq - q_split)])
+        q_pos0 = (a0, a1)
+    q = _randn((B, Sq, Hq, D), g, torch.bfloat16)
+    kbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
+    vbuf = _randn((B, sum(sks), Hkv, D), g, torch.bfloat16)
+    offs = [sum(sks[:i]) for i in range(n_ch)]
+    k_pos = torch.cat([torch.arange(starts[i], starts[i] + sks[i]) for i in range(n_ch)])
+    table, q_in = None, q
+    if rope:
+        fc = orc.precompute_freqs_cis(D, int(q_pos.max()) + 2)
+        q_in, _ = orc.apply_rotary_emb(q, q, fc[q_pos])          # what the kernel's prologue must produce
+        table = ltr.rope_table(fc.cuda())
+    o_ref, lse_ref = orc.dense_attention(q_in.float(), kbuf.float(), vbuf.float(), q_pos, k_pos, causal)
+    qd, kd, vd = _dev(q, kbuf, vbuf)
+    ks = [kd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    vs = [vd[:, offs[i]:offs[i] + sks[i]] for i in range(n_ch)]
+    got = {}
+    for rows in (256, 512):
+        q_rot = torch.full_like(qd, float("nan")) if rope else None
+        if stepwise:
+            o, lse = ltr.attn_fwd(qd, ks[:1], vs[:1], starts[:1], q_pos0, q_split, causal, out_dtype=torch.float32,
+                                  q_rope=table, q_rot_out=q_rot, fwd_rows=rows)
+            for i in range(1, n_ch):
+                ltr.attn_fwd(qd, ks[i:i + 1], vs[i:i + 1], starts[i:i + 1], q_pos0, q_split, causal, out=o, lse=lse, merge=True,
+                             q_rope=table, fwd_rows=rows)
+        else:
+            o, lse = ltr.attn_fwd(qd, ks, vs, starts, q_pos0, q_split, causal, out_dtype=out_dtype, q_rope=table,
+                                  q_rot_out=q_rot, fwd_rows=rows)
+        if rope:
+            assert torch.equal(q_rot.cpu(), q_in), (rows, seed)
+        got[rows] = (o.float().cpu(), lse.cpu())
+        assert (got[rows][0].double() - o_ref).abs().max() < O_TOL_BF16, (rows, seed)
+        fin = torch.isfinite(lse_ref)
+        assert (got[rows][1].double()[fin] - lse_ref[fin]).abs().max() < LSE_TOL_BF16, (rows, seed)
+        assert torch.isinf(got[rows][1][~fin]).all()
+    assert (got[256][0] - got[512][0]).abs().max() <= 2e-2
+    fin = torch.isfinite(got[256][1])
+    assert torch.equal(fin, torch.isfinite(got[512][1]))
+    assert (got[256][1][fin] - got[512][1][fin]).abs().max() <= 1e-3
+
+
+def test_fwd_rows_512_refused_where_it_does_not_exist(ltr):
+    g = torch.Generator().manual_seed(2)
+    q, k, v = (_randn((1, 64, 2, 128), g, torch.bfloat16).cuda() for _ in range(3))
+    with pytest.raises(RuntimeError):
+        ltr.attn_fwd(q, [k], [v], [0], fwd_rows=512)            # head dim 128
+    with pytest.raises(RuntimeError):
+        ltr.attn_fwd(q, [k], [v], [0], fwd_rows=128)
+    q, k, v = (_randn((1, 64, 2, 64), g, torch.float32).cuda() for _ in range(3))
+    with pytest.raises(RuntimeError):
+        ltr.attn_fwd(q, [k], [v], [0], fwd_rows=512)            # fp32

@@ -28,7 +28,7 @@ def test_header_symbols_exported():
     assert declared == set(L.EXPORTS), declared
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.ltr_abi_version() == 6
+    assert lib.ltr_abi_version() == 7
     assert lib.ltr_strerror(0) == b"ok" and b"aligned" in lib.ltr_strerror(-3)
 
 
