@@ -265,8 +265,8 @@ def test_config5_full_ulysses_layout(ltr):
 def test_head_dim_64_ring_share_both_block_sizes(ltr, keys, rows):
     """Head dim 64 at a size where the 256-key dK/dV blocks and 512-row dQ blocks are what the library runs: one zig-zag rank
     share (rank 2 of 4: half-chunks 2 and 5 of 8 x 2048 positions) of a causal GQA 8/2 sequence of 16384, B = 2, against all
-    8 KV half-chunks in ring order, fp32 dK / dV accumulators, bf16 dQ with DELTA from O.  Both block sizes forced through
-    the hint flags; sampled rows (O, LSE, dQ) and sampled keys (dK, dV) against the oracle's closed form."""
+    8 KV half-chunks in ring order, fp32 dK / dV accumulators, bf16 dQ with DELTA from O.  Both block sizes of all three
+    kernels forced through the hint flags (the forward with the dQ kernel's rows per block); sampled rows (O, LSE, dQ) and sampled keys (dK, dV) against the oracle's closed form."""
     g = torch.Generator().manual_seed(5)
     B, Hq, Hkv, D, S, W = 2, 8, 2, 64, 16384, 4
     hc = S // (2 * W)
@@ -285,7 +285,7 @@ def test_head_dim_64_ring_share_both_block_sizes(ltr, keys, rows):
     vs = [vd[:, i * hc:(i + 1) * hc] for i in order]
     pos0 = [i * hc for i in order]
     qp = (r * hc, (2 * W - 1 - r) * hc)
-    ol, lsel = ltr.attn_fwd(ql, ks, vs, pos0, qp, hc, True)
+    ol, lsel = ltr.attn_fwd(ql, ks, vs, pos0, qp, hc, True, fwd_rows=rows)     # the forward's block follows the dQ kernel's
     dk = torch.zeros(kd.shape, dtype=torch.float32, device="cuda")
     dv = torch.zeros(vd.shape, dtype=torch.float32, device="cuda")
     dks = [dk[:, i * hc:(i + 1) * hc] for i in order]
