@@ -298,3 +298,31 @@ def test_head_dim_64_ring_share_both_block_sizes(ltr, keys, rows):
     oc, lsec = ol.cpu(), lsel.cpu()
     _check_rows(q[:, qpos], k, v, qpos, kpos, True, oc, lsec, do, dq.cpu(), n=20)
     _check_keys(q[:, qpos], k, v, oc, lsec, do, qpos, kpos, True, dk.cpu(), dv.cpu(), n=8)
+
+
+@pytest.mark.parametrize("Sq", [2048, 1900])
+def test_head_dim_64_paired_512_row_blocks(ltr, Sq):
+    """Head dim 64, one causal chunk, enough (batch, head) pairs that the 512-row blocks of the forward and dQ kernels are
+    handed out in pairs (late q tile + early counterpart: 4 tiles -> 2 slots x 128 pairs = 256 blocks, one per CU), with a
+    ragged last tile in the second case.  512 rows forced through the hint flags (the library's own choice at 2048); sampled
+    rows and keys against the oracle's closed form."""
+    g = torch.Generator().manual_seed(11 + Sq)
+    B, Hq, Hkv, D = 4, 32, 8, 64
+    q = torch.randn(B, Sq, Hq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Sq, Hkv, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Sq, Hkv, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, Sq, Hq, D, generator=g).to(torch.bfloat16)
+    qd, kd, vd, dod = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o, lse = ltr.attn_fwd(qd, [kd], [vd], [0], 0, None, True, fwd_rows=512)
+    o256, lse256 = ltr.attn_fwd(qd, [kd], [vd], [0], 0, None, True, fwd_rows=256)
+    assert (o.float() - o256.float()).abs().max() <= 2e-2 and (lse - lse256).abs().max() <= 1e-3
+    dq = torch.empty(qd.shape, dtype=torch.bfloat16, device="cuda")
+    dk = torch.empty(kd.shape, dtype=torch.bfloat16, device="cuda")
+    dv = torch.empty(vd.shape, dtype=torch.bfloat16, device="cuda")
+    delta_ws = torch.empty(B, Hq, Sq, dtype=torch.float32, device="cuda")
+    ltr.attn_bwd_accumulate(qd, dod, lse, delta_ws, [kd], [vd], [0], dq, [dk], [dv], 0, None, True, do_dkdv=False, o=o, dq_rows=512)
+    ltr.attn_bwd_accumulate(qd, dod, lse, delta_ws, [kd], [vd], [0], dq, [dk], [dv], 0, None, True, do_dq=False)
+    pos = torch.arange(Sq)
+    oc, lsec = o.cpu(), lse.cpu()
+    _check_rows(q, k, v, pos, pos, True, oc, lsec, do, dq.cpu(), n=30)
+    _check_keys(q, k, v, oc, lsec, do, pos, pos, True, dk.float().cpu(), dv.float().cpu(), n=8)
