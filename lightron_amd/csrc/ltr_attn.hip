@@ -541,10 +541,12 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     // A slot is one q tile (late, heavier tiles first) or, when the host paired them, a late tile and its early
     // counterpart: under a causal mask every block then has the same amount of work.
     const bool paired = p.n_slots != p.n_qtiles;
+    // every other block (of an XCD) takes the early tile first: the blocks of a round then change tiles at different times
+    const bool two = paired && slot < p.n_qtiles - 1 - slot, early_first = two && ((blockIdx.x >> 3) & 1);
 #pragma nounroll
     for (int part = 0; part < 2; part++) {
-    const int qt = part == 0 ? p.n_qtiles - 1 - slot : slot;
-    if (part == 1 && (!paired || qt >= p.n_qtiles - 1 - slot)) break;
+    const int qt = (part == 0) != early_first ? p.n_qtiles - 1 - slot : slot;
+    if (part == 1 && !two) break;
     if (part == 1) __syncthreads();   // the first tile's epilogue used the LDS buffers as staging areas
     // the lane index is made opaque per tile: everything derived from it (LDS addresses of the tile loop ...) is then
     // computed inside the tile's own scope instead of being hoisted out of this loop and kept alive across the epilogue
@@ -1645,10 +1647,11 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     const int b = pair / p.Hkv, hkv = pair % p.Hkv, h = hkv * p.n_rep + rep;
     // one q tile per block (late tiles first) or a late tile and its early counterpart (see q_tile_slots)
     const bool paired = p.n_slots != n_qt;
+    const bool two = paired && slot < n_qt - 1 - slot, early_first = two && ((blockIdx.x >> 3) & 1);   // as in the forward kernel
 #pragma nounroll
     for (int part = 0; part < 2; part++) {
-    const int qt = part == 0 ? n_qt - 1 - slot : slot;
-    if (part == 1 && (!paired || qt >= n_qt - 1 - slot)) break;
+    const int qt = (part == 0) != early_first ? n_qt - 1 - slot : slot;
+    if (part == 1 && !two) break;
     if (part == 1) __syncthreads();   // the first tile's epilogue used the LDS buffers as staging areas
     int lane_of_part = threadIdx.x & 63;   // opaque per tile, see the forward kernel
     asm volatile("" : "+v"(lane_of_part));
