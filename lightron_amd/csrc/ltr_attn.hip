@@ -40,7 +40,8 @@
 //   RoPE: with LTR_ROPE_Q the forward rotates each q row in its operand registers (rope_rotate8) and can store the
 //   rotated row; with LTR_ROPE_DQ the dQ kernel's epilogue rotates dQ by the conjugate angles (rope_conj4).
 //   Block scheduling under a causal mask: a forward / dQ block takes a late q tile and its early counterpart when the
-//   host says so (q_tile_slots), and the dK/dV kernel's chunk table is sorted by position (longest blocks first).
+//   host says so (q_tile_slots; every other block in the opposite order, so that equal blocks do not all change tiles
+//   at once), and the dK/dV kernel's chunk table is sorted by position (longest blocks first).
 //   ltr_attn_bwd_noalloc keeps its DELTA workspace in the fixed __device__ array `scratch` (see there).
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, i = l % 32, h = l / 32):
