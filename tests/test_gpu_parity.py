@@ -881,7 +881,7 @@ def test_rope_sweep_bit_exact(ltr, seed):
     assert got.dtype == dtype and torch.equal(got.cpu(), ref)
 
 
-@pytest.mark.parametrize("seed", list(range(12)))
+@pytest.mark.parametrize("seed", list(range(24)))
 def test_dkdv_block_size_hints_d64(ltr, seed):
     """Head dim 64: the dK/dV kernel with 128 and with 256 keys per block (LTR_DKDV_KEYS_128 / _256, the latter two 32-key
     halves per wave), forced through the hint flags on shapes that the library's own choice would not send to the wide
@@ -997,7 +997,7 @@ def test_no_query_rows(ltr, dtype):
     assert ltr.attn_delta(o2, o2).numel() == 0
 
 
-@pytest.mark.parametrize("seed", list(range(12)))
+@pytest.mark.parametrize("seed", list(range(24)))
 def test_fwd_block_size_hints_d64(ltr, seed):
     """Head dim 64: the forward kernel with 256 and with 512 query rows per block (LTR_FWD_ROWS_256 / _512, the latter two
     32-row blocks per wave and 64-key tiles), forced through the hint flags: ragged rows and chunks, several chunks, GQA,
