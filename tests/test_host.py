@@ -138,7 +138,7 @@ def test_bench_traffic_figure_is_tied_to_the_kernel_source(tmp_path, monkeypatch
     monkeypatch.setattr(bench, "COUNTER_PROFILE", str(prof))
     val, why = bench._measured_traffic("bwd_dkdv_kernel<128, 1>")
     assert val == 1.2988e9 and digest[:12] in why
-    assert bench._measured_traffic("fwd_bf16_kernel<128>")[0] is None      # no line for that kernel
+    assert bench._measured_traffic("fwd_bf16_kernel<128, 2>")[0] is None   # no line for that kernel
     src.write_text("kernel text, edited")
     val, why = bench._measured_traffic("bwd_dkdv_kernel<128, 1>")
     assert val is None and "stale" in why
