@@ -183,9 +183,10 @@ def _device_report(la, torch, probe=True):
     """hipDeviceProp facts of the device plus what it sustains on the matrix pipe right now: a register-resident
     v_mfma_f32_32x32x16_bf16 loop on random and on constant operands, with the shader clock measured inside each."""
     import ctypes
-    lib = la._lib.load()
+    lib = la._lib.load_probe()      # the measurement library (include/ltr_probe.h), not the product
     info = la._lib.DeviceInfo()
-    la._lib.check(lib.ltr_device_info(ctypes.byref(info)), "ltr_device_info")
+    if lib.ltr_device_info(ctypes.byref(info)) != 0:
+        raise RuntimeError("ltr_device_info failed")
     rep = {"name": torch.cuda.get_device_properties(0).name, "arch": info.arch.decode(), "cus": info.compute_units,
            "clock_mhz": info.clock_khz // 1000, "memory_clock_mhz": info.memory_clock_khz // 1000,
            "memory_bus_bits": info.memory_bus_bits, "hbm_gib": round(info.hbm_bytes / 2**30, 1)}
@@ -202,7 +203,8 @@ def _device_report(la, torch, probe=True):
         for _ in range(2):      # the first launch also ramps the clock
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            la._lib.check(lib.ltr_probe_mfma(ws.data_ptr(), n, iters, rnd, stream), "ltr_probe_mfma")
+            if lib.ltr_probe_mfma(ws.data_ptr(), n, iters, rnd, stream) != 0:
+                raise RuntimeError("ltr_probe_mfma failed")
             e1.record()
             torch.cuda.synchronize()
             t = ws[:16].view(torch.int64).cpu()
@@ -257,6 +259,10 @@ def _run_attention(la, torch, cfg, steps, warmup, data="randn", min_warm_s=0.0, 
         else:
             qp, qsplit = (r * sl, r * sl), sl
         tables[r] = (ks, vs, pos, qp, qsplit)
+
+    # the kernels these launches run, as the library itself reports them (ltr_attn_plan: the function that sizes the launches)
+    ks0, _, pos0_, qp0_, qsplit0_ = tables[cfg["ranks"][0]]
+    plan = la.attn_plan(B, Hq, Hkv, D, sl, [k.shape[1] for k in ks0], pos0_, qp0_, qsplit0_, causal)
 
     o_all = torch.empty_like(q_all)
     lse_all = torch.empty(W, B, Hq, sl, dtype=torch.float32, device=dev)
@@ -339,20 +345,19 @@ def _run_attention(la, torch, cfg, steps, warmup, data="randn", min_warm_s=0.0, 
     fwd_ms = avg("fwd")
     launches = len(cfg["ranks"])
     f_share = f_fwd / launches                      # forward flops of one launch (one rank's share)
-    kernels = {"fwd_bf16_kernel": {"ms_per_launch": round(fwd_ms, 4), "algorithmic_tflops": round(f_share / fwd_ms / 1e9, 2),
-                                   "gemms_credited": 2, "gemms_executed": 2}}
+    kernels = {"fwd_bf16_kernel": {"name": plan["fwd"]["kernel"], "ms_per_launch": round(fwd_ms, 4),
+                                   "algorithmic_tflops": round(f_share / fwd_ms / 1e9, 2), "gemms_credited": 2, "gemms_executed": 2}}
     if bwd:
         # credited backward work is 5 GEMMs (S, dP, dV, dK, dQ); the dQ kernel recomputes S and dP
         dkdv_ms, dq_ms = avg("dkdv"), avg("dq")
-        kernels["bwd_dkdv_kernel"] = {"ms_per_launch": round(dkdv_ms, 4), "gemms_credited": 4, "gemms_executed": 4,
-                                      "algorithmic_tflops": round(2.0 * f_share / dkdv_ms / 1e9, 2)}
-        kernels["bwd_dq_kernel"] = {"ms_per_launch": round(dq_ms, 4), "gemms_credited": 1, "gemms_executed": 3,
+        kernels["bwd_dkdv_kernel"] = {"name": plan["dkdv"]["kernel"], "ms_per_launch": round(dkdv_ms, 4), "gemms_credited": 4,
+                                      "gemms_executed": 4, "algorithmic_tflops": round(2.0 * f_share / dkdv_ms / 1e9, 2)}
+        kernels["bwd_dq_kernel"] = {"name": plan["dq"]["kernel"], "ms_per_launch": round(dq_ms, 4), "gemms_credited": 1, "gemms_executed": 3,
                                     "algorithmic_tflops": round(0.5 * f_share / dq_ms / 1e9, 2),
                                     "executed_tflops": round(1.5 * f_share / dq_ms / 1e9, 2)}
-        # template arguments: head dim, 32-key halves per wave (2 = the 256-key blocks the library picks for long head-dim-64 streams)
-        dom, dom_ms, dom_flops = "bwd_dkdv_kernel<%d, %d>" % (D, 2 if (D == 64 and not causal and S >= 4096) else 1), dkdv_ms, 2.0 * f_share
+        dom, dom_ms, dom_flops = plan["dkdv"]["kernel"], dkdv_ms, 2.0 * f_share
     else:
-        dom, dom_ms, dom_flops = "fwd_bf16_kernel<%d, 1>" % D, fwd_ms, f_share
+        dom, dom_ms, dom_flops = plan["fwd"]["kernel"], fwd_ms, f_share
     return {"dt": dt, "f_total": f_total, "kernels": kernels, "launches": launches, "steps": steps, "warmup": n_warm,
             "dominant": (dom, dom_flops / (dom_ms * 1e-3) / 1e12)}
 
@@ -436,6 +441,203 @@ def _run_c4_rope(la, torch, steps, warmup):
             "k_pass_ms": round(t_k, 4)}
 
 
+def _run_ref_default(la, torch):
+    """The reference's own default shapes (config/config_tinystories.json:21-23 with the gpt2 model: micro-batch 4, 12
+    heads of 64, sequence 128; trainer.py:48-55 runs forward and autograd backward): one causal attention call through the
+    drop-in (block_attention, autograd) beside the library attention the reference calls there
+    (F.scaled_dot_product_attention, model/model.py:193), microseconds per forward+backward call with the host side
+    included (wall clock over many calls, one synchronisation at the end), S = 128, 256, 512."""
+    import torch.nn.functional as F
+    dev = torch.device("cuda:0")
+    B, H, D = 4, 12, 64
+    out = {"what": "us per forward+backward call, host side included, bf16 causal B=4 H=12 D=64; best of 3 interleaved runs of 300 calls"}
+
+    def wall(fn, n=300, warm=60):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    for S in (128, 256, 512):
+        g = torch.Generator().manual_seed(S)
+        q, k, v = (torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True) for _ in range(3))
+        do = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(dev)
+        qt, kt, vt = (x.detach().transpose(1, 2).requires_grad_(True) for x in (q, k, v))     # [B, H, S, D] views for SDPA
+        dot = do.transpose(1, 2)
+
+        def ours():
+            o, _ = la.block_attention(q, [k], [v], [0], causal=True)
+            o.backward(do)
+            q.grad = k.grad = v.grad = None
+
+        def library():
+            o = F.scaled_dot_product_attention(qt, kt, vt, is_causal=True)
+            o.backward(dot)
+            qt.grad = kt.grad = vt.grad = None
+
+        def ours_fwd():
+            with torch.no_grad():
+                la.block_attention(q, [k], [v], [0], causal=True)
+
+        def library_fwd():
+            with torch.no_grad():
+                F.scaled_dot_product_attention(qt, kt, vt, is_causal=True)
+
+        t = {"block_attention_us": [], "library_sdpa_us": [], "block_attention_fwd_only_us": [], "library_sdpa_fwd_only_us": []}
+        for _ in range(3):
+            t["block_attention_us"].append(wall(ours))
+            t["library_sdpa_us"].append(wall(library))
+            t["block_attention_fwd_only_us"].append(wall(ours_fwd))
+            t["library_sdpa_fwd_only_us"].append(wall(library_fwd))
+        out["S%d" % S] = {key: round(min(vals), 1) for key, vals in t.items()}
+    return out
+
+
+def _run_c3_stepwise(la, torch, steps, warmup):
+    """Config 3, one zig-zag rank share (rank 0), in the call pattern of a real ring, where KV chunks arrive one at a time:
+    the forward is one launch per half-chunk with the (O, LSE) merge fused into the kernel's epilogue (LTR_MERGE, fp32 O
+    and LSE read-modify-written by every launch after the first), the backward one ltr_attn_bwd per half-chunk adding
+    into fp32 dQ / dK / dV accumulators (DELTA from one ltr_attn_bwd_delta launch), then the casts.  Beside it the same
+    share through one launch per kernel over the 16-entry chunk table, which is what the headline times."""
+    dev = torch.device("cuda:0")
+    cfg = _workload("c3")
+    B, Hq, Hkv, D, S, W = (cfg[x] for x in ("B", "Hq", "Hkv", "D", "S", "W"))
+    sl, hc, r = S // W, S // (2 * W), 0
+    g = torch.Generator().manual_seed(0)
+    def mk(h, n):
+        return torch.randn(B, n, h, D, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v, do = mk(Hq, sl), mk(Hkv, S), mk(Hkv, S), mk(Hq, sl)
+    # the ring's visiting order (r, r-1, ... mod W), two half-chunks per rank; k / v here are stored in POSITION order
+    order = [(r - s_) % W for s_ in range(W)]
+    halves = [h_ for j in order for h_ in (j, 2 * W - 1 - j)]
+    ks = [k[:, h_ * hc:(h_ + 1) * hc] for h_ in halves]
+    vs = [v[:, h_ * hc:(h_ + 1) * hc] for h_ in halves]
+    pos = [h_ * hc for h_ in halves]
+    qp, qsplit = (r * hc, (2 * W - 1 - r) * hc), hc
+    o32 = torch.empty(B, sl, Hq, D, dtype=torch.float32, device=dev)
+    o16 = torch.empty(B, sl, Hq, D, dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(B, Hq, sl, dtype=torch.float32, device=dev)
+    dq32 = torch.empty(B, sl, Hq, D, dtype=torch.float32, device=dev)
+    dq16 = torch.empty(B, sl, Hq, D, dtype=torch.bfloat16, device=dev)
+    dk32, dv32 = torch.empty(k.shape, dtype=torch.float32, device=dev), torch.empty(v.shape, dtype=torch.float32, device=dev)
+    dks = [dk32[:, h_ * hc:(h_ + 1) * hc] for h_ in halves]
+    dvs = [dv32[:, h_ * hc:(h_ + 1) * hc] for h_ in halves]
+    delta = torch.empty(B, Hq, sl, dtype=torch.float32, device=dev)
+    n = len(ks)
+
+    def stepwise_fwd():
+        la.attn_fwd(q, ks[:1], vs[:1], pos[:1], qp, qsplit, True, out=o32, lse=lse)
+        for i in range(1, n):
+            la.attn_fwd(q, ks[i:i + 1], vs[i:i + 1], pos[i:i + 1], qp, qsplit, True, out=o32, lse=lse, merge=True)
+
+    def stepwise_bwd():
+        dq32.zero_(); dk32.zero_(); dv32.zero_()
+        d = la.attn_delta(o32, do)
+        for i in range(n):
+            la.attn_bwd_accumulate(q, do, lse, d, ks[i:i + 1], vs[i:i + 1], pos[i:i + 1], dq32, dks[i:i + 1], dvs[i:i + 1], qp, qsplit, True)
+        la.cast_to_bf16(dq32); la.cast_to_bf16(dk32); la.cast_to_bf16(dv32)
+
+    def table_fwd():
+        la.attn_fwd(q, ks, vs, pos, qp, qsplit, True, out=o16, lse=lse)
+
+    def table_bwd():
+        dk32.zero_(); dv32.zero_()
+        la.attn_bwd_accumulate(q, do, lse, delta, ks, vs, pos, dq16, dks, dvs, qp, qsplit, True, o=o16)
+        la.cast_to_bf16(dk32); la.cast_to_bf16(dv32)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    table_fwd()      # o16 / lse for the table backward
+    res = {}
+    for _ in range(2):
+        for key, fn in (("table_fwd_ms", table_fwd), ("table_bwd_ms", table_bwd), ("stepwise_fwd_ms", stepwise_fwd),
+                        ("stepwise_bwd_ms", stepwise_bwd)):
+            ms = timed(fn)
+            res[key] = min(ms, res.get(key, ms))
+    pairs = _n_pairs(cfg, r)
+    f_share = 14.0 * B * Hq * D * pairs
+    t_step, t_tab = res["stepwise_fwd_ms"] + res["stepwise_bwd_ms"], res["table_fwd_ms"] + res["table_bwd_ms"]
+    out = {"what": "config 3, rank 0's share: one launch per ring step (16 forward launches with LTR_MERGE into fp32 O/LSE, 16 "
+                   "ltr_attn_bwd calls into fp32 dQ/dK/dV, zero-fills, DELTA pass and casts included) beside one launch per "
+                   "kernel over the 16-entry chunk table",
+           "launches_per_share": {"stepwise": 16 + 1 + 2 * 16 + 6, "table": 1 + 2 + 4}}
+    out.update({key: round(val, 4) for key, val in res.items()})
+    out.update({"stepwise_ms": round(t_step, 4), "table_ms": round(t_tab, 4), "stepwise_over_table": round(t_step / t_tab, 4),
+                "stepwise_tflops": round(f_share / t_step / 1e9, 1), "table_tflops": round(f_share / t_tab / 1e9, 1)})
+    return out
+
+
+def _run_c1(la, torch):
+    """Config 1 (the reference's CPU-runnable plumbing case and its acceptance dtype: B=2, H=8, S=1024 as 4 ranks x 256,
+    D=64, fp32, causal): every rank's chunk against the chunks it sees, forward alone and forward+backward, on the fp32
+    kernels.  The whole config is 2.1e9 flop (forward), microseconds of work: it measures launches, not the matrix pipe,
+    so a larger fp32 problem (B=2, H=8, S=4096, one chunk) is timed beside it.  Fractions are of the fp32 MFMA peak."""
+    dev = torch.device("cuda:0")
+    PEAK32 = 157.3
+
+    def case(B, H, D, S, W):
+        sl = S // W
+        g = torch.Generator().manual_seed(0)
+        q, k, v, do = (torch.randn(B, S, H, D, generator=g).to(dev) for _ in range(4))
+        o = torch.empty_like(q)
+        lse = torch.empty(W, B, H, sl, dtype=torch.float32, device=dev)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        tabs = []
+        for r in range(W):
+            order = [(r - s_) % W for s_ in range(W)]
+            tabs.append(([k[:, j * sl:(j + 1) * sl] for j in order], [v[:, j * sl:(j + 1) * sl] for j in order],
+                         [j * sl for j in order], [dk[:, j * sl:(j + 1) * sl] for j in order], [dv[:, j * sl:(j + 1) * sl] for j in order]))
+
+        def fwd():
+            for r in range(W):
+                ks, vs, pos, _, _ = tabs[r]
+                la.attn_fwd(q[:, r * sl:(r + 1) * sl], ks, vs, pos, r * sl, None, True, out=o[:, r * sl:(r + 1) * sl], lse=lse[r])
+
+        def fwd_bwd():
+            fwd()
+            dq.zero_(); dk.zero_(); dv.zero_()
+            for r in range(W):
+                ks, vs, pos, dks, dvs = tabs[r]
+                rows = slice(r * sl, (r + 1) * sl)
+                d = la.attn_delta(o[:, rows], do[:, rows])
+                la.attn_bwd_accumulate(q[:, rows], do[:, rows], lse[r], d, ks, vs, pos, dq[:, rows], dks, dvs, r * sl, None, True)
+
+        def timed(fn, min_s=0.2):
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+            n, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < min_s:
+                for _ in range(10):
+                    fn()
+                n += 10
+                torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / n
+        f_fwd = 4.0 * B * H * D * (S * (S + 1) // 2)
+        t_f, t_fb = timed(fwd), timed(fwd_bwd)
+        plan = la.attn_plan(B, H, H, D, sl, [sl] * W, [j * sl for j in range(W)], (W - 1) * sl, None, True, dtype=torch.float32)
+        return {"fwd_us": round(t_f * 1e6, 1), "fwd_tflops": round(f_fwd / t_f / 1e12, 3), "fwd_frac_of_fp32_mfma_peak": round(f_fwd / t_f / 1e12 / PEAK32, 4),
+                "fwd_bwd_us": round(t_fb * 1e6, 1), "fwd_bwd_tflops": round(3.5 * f_fwd / t_fb / 1e12, 3),
+                "fwd_bwd_frac_of_fp32_mfma_peak": round(3.5 * f_fwd / t_fb / 1e12 / PEAK32, 4), "fwd_kernel": plan["fwd"]["kernel"]}
+
+    return {"what": "fp32 path; config 1 = B=2 H=8 S=1024 (4 ranks x 256) D=64 causal, 4 launches per pass; large = B=2 H=8 S=4096 D=64 causal, one chunk",
+            "fp32_mfma_peak_tflops": PEAK32, "config1": case(2, 8, 64, 1024, 4), "large": case(2, 8, 64, 4096, 1)}
+
+
 def _bench_mfma_ceiling(args):
     """What the device sustains on the matrix pipe, for the record beside the attention numbers: the register-resident
     MFMA loop of ltr_probe_mfma on random and constant operands with the shader clock of each, and the vendor library's
@@ -466,55 +668,12 @@ def _bench_mfma_ceiling(args):
     print(json.dumps(out), flush=True)
 
 
-def _bench_dq_atomics(args):
-    """The rate at which 64 x 128 fp32 partial dQ tiles can be added into memory with global atomics (ltr_probe_atomic_tile_add):
-    what a backward that produced dQ inside the key-owning blocks would need, beside what it needs at the dK/dV kernel's
-    speed."""
-    import torch
-    import lightron_amd as la
-    torch.cuda.set_device(0)
-    lib = la._lib.load()
-    n = 8192 + (1 << 20)
-    g = torch.Generator().manual_seed(1)
-    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
-    ws[8192:] = ((torch.rand((n - 8192) // 2, generator=g) * 4 - 2).to(torch.bfloat16)).view(torch.uint8).cuda()
-    dst = torch.zeros(32, 4096, 128, dtype=torch.float32, device="cuda")
-    stream = torch.cuda.current_stream().cuda_stream
-    steps = 512
-    res = {}
-    for key, with_mfma in (("atomic_adds_only", 0), ("atomic_adds_between_40_mfma_per_wave", 1)):
-        best = None
-        for _ in range(3):
-            dst.zero_()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            la._lib.check(lib.ltr_probe_atomic_tile_add(dst.data_ptr(), dst.numel(), ws.data_ptr(), n, steps, with_mfma, stream),
-                          "ltr_probe_atomic_tile_add")
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            best = ms if best is None or ms < best else best
-        ok = bool((dst == steps / 8).all().item())
-        res[key] = {"ms": round(best, 3), "us_per_tile_per_block": round(best * 1e3 / steps, 3),
-                    "payload_TB_per_s": round(256 * steps * 32768 / (best * 1e-3) / 1e12, 3), "sums_correct": ok}
-    # MFMA-only time of the same loop, for the share of the adds in the combined run: 40 MFMA per wave and step
-    need = {"step_us_at_dkdv_speed": 2.06, "payload_TB_per_s_needed": round(256 * 32768 / 2.06e-6 / 1e12, 2),
-            "note": "a 5-GEMM step of 64 rows x 128 keys x 4 slices per CU takes about 2.06 us at 1300 TFLOP/s; one 32 KiB tile add per step"}
-    out = {"metric": "fp32 global-atomic tile-add rate (partial dQ of a fused backward)", "value": res["atomic_adds_only"]["payload_TB_per_s"],
-           "unit": "TB/s", "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
-           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "256 blocks x 8 waves, each block adds one 64 x 128 fp32 tile per step into a [32, 4096, 128] buffer shared like dQ"},
-           "results": res, "needed_by_a_fused_backward": need}
-    print(json.dumps(out), flush=True)
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling", "dq_atomics"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other workloads and the device probe")
     args = ap.parse_args()
@@ -528,8 +687,6 @@ def main():
         return _bench_rope(args)
     if args.workload == "mfma_ceiling":
         return _bench_mfma_ceiling(args)
-    if args.workload == "dq_atomics":
-        return _bench_dq_atomics(args)
     la._lib.load()
     torch.cuda.set_device(0)
     cfg = _workload(args.workload)
@@ -573,6 +730,11 @@ def main():
                             "dominant_kernel_frac": round(r["dominant"][1] / MFMA_BF16_PEAK_TFLOPS, 4)}
         torch.cuda.empty_cache()
         others["c4_rope"] = _run_c4_rope(la, torch, 5, 2)
+        torch.cuda.empty_cache()
+        others["c3_stepwise"] = _run_c3_stepwise(la, torch, 5, 2)
+        torch.cuda.empty_cache()
+        others["c1"] = _run_c1(la, torch)
+        others["ref_default"] = _run_ref_default(la, torch)
         out["other_workloads"] = others
         torch.cuda.empty_cache()
         out["data_dependence"] = _data_dependence(la, torch, cfg)

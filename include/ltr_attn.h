@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define LTR_ABI_VERSION 7
+#define LTR_ABI_VERSION 8
 #define LTR_MAX_CHUNKS 32
 
 /* element types */
@@ -262,47 +262,26 @@ typedef struct ltr_rope_args {
 int ltr_rope_apply(const ltr_rope_args *args, void *stream);
 
 /*
- * Measurement helpers (no counterpart in the reference: its only performance output is a printed wall time,
- * ring_attention.py:195-196).  A benchmark prints the kernels' rates beside what the device itself sustains.
- *
- * ltr_device_info - facts of the CURRENT device as hipDeviceProp reports them (host call, nothing is enqueued).
- *
- * ltr_probe_mfma - enqueues one kernel in which every wave of every CU (one block of 8 waves per CU) runs
- * 4 * iters v_mfma_f32_32x32x16_bf16 on register-resident operands: the device's matrix-pipe ceiling.
- * random_operands != 0: the operands are read once from workspace bytes [8192, workspace_bytes), which the caller
- * fills (random bf16 data makes the chip run at the clock its power limit allows); 0: constant operands.
- * Results, valid once the stream has finished: ((int64_t *)workspace)[0] = ticks of the constant 100 MHz wall clock
- * that ONE wave's loop took, [1] = ticks of the shader clock counter over the same interval: their ratio is the shader
- * clock under this load.  (The two waves of a SIMD do not alternate - the older one runs its loop at the pipe's full rate,
- * then the other - so the rate is taken over the launch's duration, timed by the caller with events on the stream:
- * CUs * 8 * iters * 4 * 32768 flop / seconds.)
- * workspace: device memory, 16-byte aligned, at least LTR_PROBE_MIN_WORKSPACE bytes.
+ * ltr_attn_plan - which kernels, with which block sizes, ltr_attn_fwd and ltr_attn_bwd would launch for this problem
+ * on the CURRENT device (host call: nothing is enqueued and no pointer in args is read; without a device the answer is
+ * for 256 compute units).  It has no counterpart in the reference (which leaves the choice of kernel to the library
+ * behind F.scaled_dot_product_attention, model/model.py:193); it is for benchmarks and profiles that must name the kernel
+ * they measured, and for tests of the size hints.  The sizes, strides' owner shapes, positions, chunk lengths, dtype and
+ * flags of args are read; flags may also carry the forward's hints (LTR_FWD_ROWS_256 / LTR_FWD_ROWS_512).  The library's
+ * launches and this answer come from one function, so they cannot drift apart.  Kernel names are those a profiler shows.
  */
-typedef struct ltr_device_info_t {
-    int32_t compute_units;
-    int32_t clock_khz;            /* hipDeviceProp.clockRate: the engine clock the device advertises */
-    int32_t memory_clock_khz;
-    int32_t memory_bus_bits;
-    int64_t lds_bytes_per_block;
-    int64_t hbm_bytes;
-    char arch[64];
-} ltr_device_info_t;
+typedef struct ltr_attn_plan_t {
+    int32_t compute_units;   /* CUs the choices were made for */
+    int32_t fwd_rows;        /* query rows per block of the forward kernel */
+    int32_t fwd_paired;      /* 1: a block takes a late q tile and its early counterpart (causal balance) */
+    int32_t dq_rows;         /* query rows per block of the dQ kernel */
+    int32_t dq_paired;
+    int32_t dkdv_keys;       /* keys per block of the dK/dV kernel */
+    int64_t fwd_blocks, dq_blocks, dkdv_blocks;
+    char fwd_kernel[48], dq_kernel[48], dkdv_kernel[48];
+} ltr_attn_plan_t;
 
-#define LTR_PROBE_MIN_WORKSPACE (8192 + 65536)
-
- /*
- * ltr_probe_atomic_tile_add - the rate at which blocks can ADD 64 x 128 fp32 tiles into shared memory with global
- * atomics: what a backward that produced dQ inside the key-owning blocks would have to sustain (one tile per block
- * per 64-row step; at the attention kernels' speed that is one every ~2 us per CU, ~4 TB/s of fp32 payload over the
- * device).  256 blocks of 8 waves; every block adds `steps` tiles (value 1.0 per element, coalesced: a half-wave = 128
- * contiguous bytes of one row) into dst, fp32 [32][4096][128], zero-filled by the caller: afterwards every element
- * holds steps / 8 (steps a multiple of 256).  with_mfma != 0: 40 MFMAs per wave between two adds, the matrix work of
- * such a step.  workspace as for ltr_probe_mfma (operands from bytes [8192, ...)).  Timed by the caller with events.
- */
-int ltr_device_info(ltr_device_info_t *out);
-int ltr_probe_mfma(void *workspace, int64_t workspace_bytes, int32_t iters, int32_t random_operands, void *stream);
-int ltr_probe_atomic_tile_add(float *dst, int64_t dst_elems, void *workspace, int64_t workspace_bytes, int32_t steps,
-                              int32_t with_mfma, void *stream);
+int ltr_attn_plan(const ltr_attn_bwd_args *args, ltr_attn_plan_t *out);
 
 int ltr_abi_version(void);
 const char *ltr_strerror(int code);

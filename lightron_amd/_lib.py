@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 # LTR_ATTN_LIB names another build of the same library (same ABI version), e.g. to compare two builds in one session
 LIB_PATH = os.environ.get("LTR_ATTN_LIB") or os.path.join(HERE, "csrc", "libltr_attn.so")
 
-LTR_ABI_VERSION = 7
+LTR_ABI_VERSION = 8
 LTR_MAX_CHUNKS = 32
 LTR_NOALLOC_MAX_ROWS = 1 << 20
 LTR_BF16, LTR_F32 = 0, 1
@@ -18,8 +18,11 @@ LTR_DKDV_KEYS_128, LTR_DKDV_KEYS_256 = 512, 1024
 LTR_DQ_ROWS_256, LTR_DQ_ROWS_512 = 2048, 4096
 LTR_FWD_ROWS_256, LTR_FWD_ROWS_512 = 8192, 16384
 
-EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_cast_f32_to_bf16", "ltr_rope_apply",
-           "ltr_device_info", "ltr_probe_mfma", "ltr_probe_atomic_tile_add", "ltr_abi_version", "ltr_strerror")
+EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_attn_plan", "ltr_cast_f32_to_bf16",
+           "ltr_rope_apply", "ltr_abi_version", "ltr_strerror")
+# the bench-only measurement library (include/ltr_probe.h); not part of the attention path
+PROBE_LIB_PATH = os.path.join(HERE, "csrc", "libltr_probe.so")
+PROBE_EXPORTS = ("ltr_device_info", "ltr_probe_mfma")
 
 _i64x3 = ctypes.c_int64 * 3
 _i64x2 = ctypes.c_int64 * 2
@@ -80,9 +83,17 @@ class DeviceInfo(ctypes.Structure):
                 ("arch", ctypes.c_char * 64)]
 
 
+class AttnPlan(ctypes.Structure):
+    _fields_ = [("compute_units", ctypes.c_int32), ("fwd_rows", ctypes.c_int32), ("fwd_paired", ctypes.c_int32),
+                ("dq_rows", ctypes.c_int32), ("dq_paired", ctypes.c_int32), ("dkdv_keys", ctypes.c_int32),
+                ("fwd_blocks", ctypes.c_int64), ("dq_blocks", ctypes.c_int64), ("dkdv_blocks", ctypes.c_int64),
+                ("fwd_kernel", ctypes.c_char * 48), ("dq_kernel", ctypes.c_char * 48), ("dkdv_kernel", ctypes.c_char * 48)]
+
+
 LTR_PROBE_MIN_WORKSPACE = 8192 + 65536
 
 _lib = None
+_probe = None
 
 
 def load():
@@ -107,13 +118,8 @@ def load():
     lib.ltr_cast_f32_to_bf16.restype = ctypes.c_int
     lib.ltr_rope_apply.argtypes = [ctypes.POINTER(RopeArgs), ctypes.c_void_p]
     lib.ltr_rope_apply.restype = ctypes.c_int
-    lib.ltr_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
-    lib.ltr_device_info.restype = ctypes.c_int
-    lib.ltr_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
-    lib.ltr_probe_mfma.restype = ctypes.c_int
-    lib.ltr_probe_atomic_tile_add.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32,
-                                              ctypes.c_int32, ctypes.c_void_p]
-    lib.ltr_probe_atomic_tile_add.restype = ctypes.c_int
+    lib.ltr_attn_plan.argtypes = [ctypes.POINTER(BwdArgs), ctypes.POINTER(AttnPlan)]
+    lib.ltr_attn_plan.restype = ctypes.c_int
     lib.ltr_abi_version.argtypes = []
     lib.ltr_abi_version.restype = ctypes.c_int
     lib.ltr_strerror.argtypes = [ctypes.c_int]
@@ -122,6 +128,22 @@ def load():
         raise RuntimeError("lightron_amd: ABI version mismatch (library %d, binding %d)"
                            % (lib.ltr_abi_version(), LTR_ABI_VERSION))
     _lib = lib
+    return lib
+
+
+def load_probe():
+    """The measurement library of bench.py (device facts, matrix-pipe ceiling probe); raises if it has not been built."""
+    global _probe
+    if _probe is not None:
+        return _probe
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise RuntimeError("lightron_amd: %s is missing - build it with `python -m lightron_amd.build`" % PROBE_LIB_PATH)
+    lib = ctypes.CDLL(PROBE_LIB_PATH)
+    lib.ltr_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
+    lib.ltr_device_info.restype = ctypes.c_int
+    lib.ltr_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+    lib.ltr_probe_mfma.restype = ctypes.c_int
+    _probe = lib
     return lib
 
 

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import threading
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -17,8 +18,33 @@ from . import _lib
 _DT = {torch.bfloat16: _lib.LTR_BF16, torch.float32: _lib.LTR_F32}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(dev) -> int:
+    """hipStream_t of torch's current stream on `dev`, as an integer."""
+    if _raw_stream is not None:
+        return _raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(dev):
+    """Context in which `dev` is the current device: the library launches on the CURRENT device.  The common case (it
+    already is) costs one query instead of a device switch and back."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(dev)
 
 
 def _s3(t: torch.Tensor):
@@ -38,11 +64,24 @@ def _same_strides(ts: Sequence[torch.Tensor]) -> bool:
     return all(t.stride() == s0 for t in ts)
 
 
+_warned_repack = False
+
+
 def _common_layout(ts):
-    """Chunks whose strides differ (separate tensors of unequal length have different batch strides) are
-    packed once into one [B, sum S, H, D] buffer and returned as its sequence slices, which share one triple."""
-    if _same_strides(ts):
+    """The ABI carries ONE stride triple for all K chunks (and one for all V chunks).  Chunks that already share it -
+    slices of one tensor along the sequence, or separate tensors of equal shape - pass through untouched.  Chunks whose
+    strides differ (separate tensors of unequal length have different batch strides) take the SLOW PATH: they are
+    copied into one [B, sum S, H, D] buffer (torch.cat: a pass over every chunk, in the forward and again in the
+    backward) and returned as its sequence slices.  Warns once per process; callers on a hot path should hand in slices
+    of one buffer."""
+    if len(ts) == 1 or _same_strides(ts):
         return list(ts)
+    global _warned_repack
+    if not _warned_repack:
+        _warned_repack = True
+        import warnings
+        warnings.warn("lightron_amd: KV chunks with different strides are packed into one buffer on every call "
+                      "(a copy of every chunk); pass sequence slices of one tensor to avoid it", stacklevel=3)
     buf = torch.cat([t for t in ts], dim=1)
     out, start = [], 0
     for t in ts:
@@ -128,7 +167,7 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
         raise RuntimeError("q_rot_out needs q_rope")
     stream = _stream_ptr(q.device)
     n = len(ks)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         for start in range(0, n, _lib.LTR_MAX_CHUNKS):
             stop = min(n, start + _lib.LTR_MAX_CHUNKS)
             a.n_chunks = stop - start
@@ -154,7 +193,7 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
     a.B, a.Hq, a.D, a.Sq = B, Hq, D, Sq
     a.o_stride, a.do_stride = _s3(o), _s3(do)
     a.o_dtype, a.do_dtype = _DT[o.dtype], _DT[do.dtype]
-    with torch.cuda.device(o.device):
+    with _on_device(o.device):
         _lib.check(lib.ltr_attn_bwd_delta(ctypes.byref(a), _stream_ptr(o.device)), "ltr_attn_bwd_delta")
     return delta
 
@@ -244,7 +283,7 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     base_flags = a.flags
     stream = _stream_ptr(q.device)
     n = len(ks)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         for start in range(0, n, _lib.LTR_MAX_CHUNKS):
             stop = min(n, start + _lib.LTR_MAX_CHUNKS)
             a.n_chunks = stop - start
@@ -260,12 +299,42 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
                 _lib.check(lib.ltr_attn_bwd(ctypes.byref(a), stream), "ltr_attn_bwd")
 
 
+def attn_plan(B: int, Hq: int, Hkv: int, D: int, Sq: int, chunk_lens: Sequence[int], k_pos0: Sequence[int], q_pos0=0,
+              q_split: Optional[int] = None, causal: bool = False, dtype: torch.dtype = torch.bfloat16, fwd_rows=None,
+              dq_rows=None, dkdv_keys=None) -> dict:
+    """Which kernels the library would launch for this problem on the current device (ltr_attn_plan: a host call, no
+    tensors needed; at most 32 chunks = one launch): block sizes, block counts and the kernels' names as a profiler
+    shows them.  fwd_rows / dq_rows / dkdv_keys force a size like the arguments of attn_fwd / attn_bwd_accumulate."""
+    lib = _lib.load()
+    a = _lib.BwdArgs()
+    a.B, a.Hq, a.Hkv, a.D, a.Sq, a.n_chunks = B, Hq, Hkv, D, Sq, len(chunk_lens)
+    a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
+    a.io_dtype = _DT[dtype]
+    a.flags = _lib.LTR_CAUSAL if causal else 0
+    for val, lo, hi, name in ((fwd_rows, _lib.LTR_FWD_ROWS_256, _lib.LTR_FWD_ROWS_512, "fwd_rows"),
+                              (dq_rows, _lib.LTR_DQ_ROWS_256, _lib.LTR_DQ_ROWS_512, "dq_rows"),
+                              (dkdv_keys, _lib.LTR_DKDV_KEYS_128, _lib.LTR_DKDV_KEYS_256, "dkdv_keys")):
+        if val is not None:
+            sizes = (128, 256) if name == "dkdv_keys" else (256, 512)
+            if val not in sizes:
+                raise RuntimeError("%s must be None, %d or %d" % ((name,) + sizes))
+            a.flags |= lo if val == sizes[0] else hi
+    for i, (sk, p0) in enumerate(zip(chunk_lens, k_pos0)):
+        a.chunk[i].sk, a.chunk[i].pos0 = int(sk), int(p0)
+    out = _lib.AttnPlan()
+    _lib.check(lib.ltr_attn_plan(ctypes.byref(a), ctypes.byref(out)), "ltr_attn_plan")
+    return {"compute_units": out.compute_units,
+            "fwd": {"kernel": out.fwd_kernel.decode(), "rows": out.fwd_rows, "paired": bool(out.fwd_paired), "blocks": out.fwd_blocks},
+            "dq": {"kernel": out.dq_kernel.decode(), "rows": out.dq_rows, "paired": bool(out.dq_paired), "blocks": out.dq_blocks},
+            "dkdv": {"kernel": out.dkdv_kernel.decode(), "keys": out.dkdv_keys, "blocks": out.dkdv_blocks}}
+
+
 def cast_to_bf16(src: torch.Tensor) -> torch.Tensor:
     lib = _lib.load()
     if src.dtype != torch.float32 or not src.is_contiguous():
         raise RuntimeError("cast_to_bf16 needs a contiguous fp32 tensor")
     dst = torch.empty(src.shape, dtype=torch.bfloat16, device=src.device)
-    with torch.cuda.device(src.device):
+    with _on_device(src.device):
         _lib.check(lib.ltr_cast_f32_to_bf16(src.data_ptr(), dst.data_ptr(), src.numel(), _stream_ptr(src.device)),
                    "ltr_cast_f32_to_bf16")
     return dst
@@ -347,6 +416,130 @@ class BlockAttentionFunction(torch.autograd.Function):
         return (dq, None, None, None, None, None, None, None, None, None, None, *dks, *dvs)
 
 
+class _PreparedCalls(threading.local):
+    """Per-thread cache of filled-in argument blocks, keyed by everything but the pointers: a training loop calls with
+    the same shapes, strides and positions every step, and then only the pointers are rewritten (autograd runs the
+    backward on another thread than the forward, and two threads must not share one block)."""
+
+    def __init__(self):
+        self.fwd, self.bwd = {}, {}
+
+
+_prepared = _PreparedCalls()
+_PREPARED_MAX = 256
+
+
+def _single_key(q, k, v, extra):
+    return (q.shape, q.stride(), k.shape, k.stride(), v.shape, v.stride(), k.dtype, v.dtype, q.device, k.device, v.device, extra)
+
+
+class SingleChunkAttentionFunction(torch.autograd.Function):
+    """block_attention for its most frequent shape - ONE KV chunk, bf16, one launch (the SDPA call sites of the reference,
+    model/model.py:193-198 and parallel/parallel_cp.py:224-229) - with the host work cut to what such a call needs:
+    the checks are made when a geometry is first seen and the argument block is kept; later calls write five pointers
+    into it.  Same kernels, same results as BlockAttentionFunction."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, meta):
+        k_pos0, q_pos0, q_split, causal, scale, q_rope = meta
+        lib = _lib.load()
+        B, Sq, Hq, D = q.shape
+        dev = q.device
+        o = torch.empty((B, Sq, Hq, D), dtype=torch.bfloat16, device=dev)
+        lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)
+        q_rot = None
+        key = _single_key(q, k, v, (k_pos0, q_pos0, q_split, causal, scale, None if q_rope is None else q_rope.shape[0]))
+        prep = _prepared.fwd.get(key)
+        if prep is None:
+            for t, name in ((q, "q"), (k, "k"), (v, "v")):
+                _req(t, name)
+            if (k.dtype != q.dtype or v.dtype != q.dtype or k.shape != v.shape or k.shape[0] != B or k.shape[3] != D
+                    or k.device != dev or v.device != dev):
+                raise RuntimeError("k/v chunk shape, dtype or device mismatch")
+            a = _lib.FwdArgs()
+            a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, k.shape[2], D, Sq
+            a.q_stride, a.o_stride, a.k_stride, a.v_stride = _s3(q), _s3(o), _s3(k), _s3(v)
+            a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
+            a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
+            a.io_dtype = a.o_dtype = _lib.LTR_BF16
+            a.n_chunks = 1
+            a.flags = (_lib.LTR_CAUSAL if causal else 0) | (_lib.LTR_ROPE_Q if q_rope is not None else 0)
+            ch = a.chunk[0]
+            ch.sk, ch.pos0 = k.shape[1], int(k_pos0)
+            if q_rope is not None:
+                a.rope_pos0, a.rope_len = 0, q_rope.shape[0]
+                a.q_rot_stride = _s3(o)          # q_rot is allocated like o: contiguous [B, Sq, Hq, D]
+            if len(_prepared.fwd) >= _PREPARED_MAX:
+                _prepared.fwd.clear()
+            prep = _prepared.fwd[key] = (a, ch, ctypes.byref(a))
+        a, ch, ref = prep
+        a.q, a.o, a.lse = q.data_ptr(), o.data_ptr(), lse.data_ptr()
+        ch.k, ch.v = k.data_ptr(), v.data_ptr()
+        if q_rope is not None:
+            _rope_table_check(q_rope, D, dev)    # the table is a per-call pointer: checked on every call
+            q_rot = torch.empty((B, Sq, Hq, D), dtype=torch.bfloat16, device=dev)
+            a.rope_freqs, a.q_rot = q_rope.data_ptr(), q_rot.data_ptr()
+        if Sq:
+            with _on_device(dev):
+                rc = lib.ltr_attn_fwd(ref, _stream_ptr(dev))
+            if rc:
+                _lib.check(rc, "ltr_attn_fwd")
+        ctx.save_for_backward(q if q_rot is None else q_rot, k, v, o, lse)
+        ctx.meta = meta
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, _dlse):
+        q, k, v, o, lse = ctx.saved_tensors
+        k_pos0, q_pos0, q_split, causal, scale, q_rope = ctx.meta
+        lib = _lib.load()
+        B, Sq, Hq, D = q.shape
+        dev = q.device
+        if do.dtype != torch.bfloat16:
+            do = do.to(torch.bfloat16)
+        if do.stride(3) != 1:
+            do = do.contiguous()
+        dq = torch.empty((B, Sq, Hq, D), dtype=torch.bfloat16, device=dev)
+        dk = torch.empty(k.shape, dtype=torch.bfloat16, device=dev)
+        dv = torch.empty(k.shape, dtype=torch.bfloat16, device=dev)
+        if Sq == 0:
+            return dq, dk.zero_(), dv.zero_(), None
+        delta = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)   # workspace: filled by the dQ kernel from o
+        key = _single_key(q, k, v, (do.stride(), k_pos0, q_pos0, q_split, causal, scale, None if q_rope is None else q_rope.shape[0]))
+        prep = _prepared.bwd.get(key)
+        if prep is None:
+            _req(do, "dO")
+            a = _lib.BwdArgs()
+            a.B, a.Hq, a.Hkv, a.D, a.Sq = B, Hq, k.shape[2], D, Sq
+            a.q_stride, a.do_stride, a.dq_stride, a.o_stride = _s3(q), _s3(do), _s3(dq), _s3(o)
+            a.k_stride, a.v_stride, a.dk_stride, a.dv_stride = _s3(k), _s3(v), _s3(dk), _s3(dv)
+            a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
+            a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
+            a.io_dtype = _lib.LTR_BF16
+            a.n_chunks = 1
+            # one call holds every key these rows see and every row that sees these keys: the kernels write bf16 results
+            a.flags = ((_lib.LTR_CAUSAL if causal else 0) | _lib.LTR_DQ_BF16 | _lib.LTR_DKDV_BF16 | _lib.LTR_DELTA_FROM_O
+                       | (_lib.LTR_ROPE_DQ if q_rope is not None else 0))
+            ch = a.chunk[0]
+            ch.sk, ch.pos0 = k.shape[1], int(k_pos0)
+            if q_rope is not None:
+                a.rope_pos0, a.rope_len = 0, q_rope.shape[0]
+            if len(_prepared.bwd) >= _PREPARED_MAX:
+                _prepared.bwd.clear()
+            prep = _prepared.bwd[key] = (a, ch, ctypes.byref(a))
+        a, ch, ref = prep
+        a.q, a.d_o, a.lse, a.delta, a.dq, a.o = q.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(), dq.data_ptr(), o.data_ptr()
+        ch.k, ch.v, ch.dk, ch.dv = k.data_ptr(), v.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        if q_rope is not None:
+            a.rope_freqs = q_rope.data_ptr()
+        with _on_device(dev):
+            rc = lib.ltr_attn_bwd(ref, _stream_ptr(dev))
+        if rc:
+            _lib.check(rc, "ltr_attn_bwd")
+        return dq, dk, dv, None
+
+
 def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, scale=None, stepwise=False,
                     out_dtype=None, kv_grad_acc=None, q_rope=None):
     """Differentiable entry: returns (O, LSE).  q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table indexed by global
@@ -357,6 +550,11 @@ def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, sca
     accumulators makes the one final cast.  That is how a ring sums dK / dV over its ranks without a bf16 rounding
     per rank."""
     n = len(ks)
+    if (n == 1 and kv_grad_acc is None and not stepwise and q.dtype == torch.bfloat16 and out_dtype in (None, torch.bfloat16)
+            and q.is_cuda and ks[0].is_cuda and vs[0].is_cuda):
+        if isinstance(q_pos0, (tuple, list)):
+            q_pos0 = (int(q_pos0[0]), int(q_pos0[1]))
+        return SingleChunkAttentionFunction.apply(q, ks[0], vs[0], (int(k_pos0[0]), q_pos0, q_split, bool(causal), scale, q_rope))
     if kv_grad_acc is not None:
         dk_accs, dv_accs = kv_grad_acc
         if len(dk_accs) != n or len(dv_accs) != n:

@@ -49,6 +49,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <math.h>
+#include <stdio.h>
 #include <type_traits>
 #include <atomic>
 #include <algorithm>
@@ -2117,6 +2118,7 @@ constexpr int LTR_MAX_DEVICES = 64;
 struct DeviceState {
     std::atomic<int> arch{0};          // 0 unknown, 1 gfx950, -1 something else
     std::atomic<int> large_lds{0};     // 1: the kernels of this device may use more than 64 KB of dynamic LDS
+    std::atomic<int> cus{0};           // compute units (0: not asked yet)
     std::atomic<float *> scratch{nullptr};   // device address of this device's copy of `scratch`
 };
 DeviceState g_dev[LTR_MAX_DEVICES];
@@ -2193,11 +2195,29 @@ double cu_fill(long long blocks, int cus) {
     return rounds > 0 ? (double)blocks / (double)(rounds * cus) : 0.0;
 }
 
-// compute units of the current device (the launch heuristics below count rounds of blocks over them)
+// compute units of the current device (the launch heuristics below count rounds of blocks over them); asked once per
+// device.  Without a device (a host-only ltr_attn_plan call) the answer is that of the part this library is written for.
 int device_cus() {
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    return cus > 0 ? cus : 256;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LTR_MAX_DEVICES) {
+        (void)hipGetLastError();   // "no device" is an answer here, not an error to leave behind
+        return 256;
+    }
+    int cus = g_dev[dev].cus.load(std::memory_order_acquire);
+    if (cus <= 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 256;
+        g_dev[dev].cus.store(cus, std::memory_order_release);
+    }
+    return cus;
+}
+
+// One kernel launch whose own status is what is returned: hipLaunchKernel reports the submission of THIS launch, so an
+// error that unrelated earlier work left in the thread's last-error slot is neither reported as ours nor cleared.
+template <class Params>
+int launch(const void *kernel, long long blocks, int threads, size_t lds_bytes, hipStream_t st, const Params &p) {
+    void *args[] = {(void *)&p};
+    return hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3((unsigned)threads), args, lds_bytes, st) == hipSuccess ? LTR_OK
+                                                                                                                      : LTR_ELAUNCH;
 }
 
 // Keys that the q rows [r0, r1] walk through under the causal mask: per chunk, those up to the rows' last position.
@@ -2233,6 +2253,113 @@ int q_tile_slots(int n_qtiles, long long blocks_per_tile, bool uneven) {
     const int n_slots = (n_qtiles + 1) / 2;
     const long long n = n_slots * blocks_per_tile, rounds = (n + cus - 1) / cus;
     return n * 10 >= rounds * cus * 9 ? n_slots : n_qtiles;
+}
+
+// What a forward launch looks like: rows per block, q tiles, slots (see q_tile_slots), blocks.  One function decides for
+// ltr_attn_fwd and for ltr_attn_plan, so the plan a caller is shown is the launch it gets.
+struct FwdPlan {
+    bool wide;          // 512-row blocks (two 32-row blocks per wave, head dim 64)
+    int rows, n_qtiles, n_slots;
+    long long blocks;
+};
+FwdPlan plan_fwd(int D, bool f32, unsigned flags, int B, int Hq, int Sq, int q_split, const int *q_pos0, const ChunkDev *chunk,
+                 int n_chunks) {
+    FwdPlan pl;
+    if (f32) {
+        pl.wide = false;
+        pl.rows = 64;
+        pl.n_qtiles = pl.n_slots = (Sq + 63) / 64;
+        pl.blocks = (long long)pl.n_qtiles * B * Hq;
+        return pl;
+    }
+    const bool causal_ = (flags & LTR_CAUSAL) != 0;
+    // query rows per block: 512 (two 32-row blocks per wave, 64-key tiles) pays at head dim 64 under the conditions of
+    // the dQ kernel's 512-row blocks (see plan_bwd)
+    bool wide = (flags & LTR_FWD_ROWS_512) != 0;
+    if (!wide && !(flags & LTR_FWD_ROWS_256) && D == 64) {
+        const int tiles512 = (Sq + 511) / 512;
+        const int slots512 = q_tile_slots(tiles512, (long long)B * Hq, causal_ && q_tiles_uneven(Sq, 512, q_split, q_pos0, chunk, n_chunks));
+        const long long blocks512 = (long long)slots512 * B * Hq, blocks256 = (long long)((Sq + 255) / 256) * B * Hq;
+        const int cus = device_cus();
+        wide = causal_ ? (Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus)
+                       : (cu_fill(blocks512, cus) * 1.07 >= cu_fill(blocks256, cus));
+    }
+    pl.wide = wide;
+    pl.rows = wide ? 512 : 256;
+    pl.n_qtiles = (Sq + pl.rows - 1) / pl.rows;
+    pl.n_slots = q_tile_slots(pl.n_qtiles, (long long)B * Hq, causal_ && q_tiles_uneven(Sq, pl.rows, q_split, q_pos0, chunk, n_chunks));
+    pl.blocks = (long long)pl.n_slots * B * Hq;
+    return pl;
+}
+
+// The same for the two backward kernels.
+struct BwdPlan {
+    bool wide_kv;       // dK/dV kernel: 256 keys per block (two 32-key halves per wave, head dim 64)
+    int keys_per_block;
+    long long kv_tiles; // key blocks over all chunks of one (batch, kv head)
+    long long kv_blocks;
+    bool wide_q;        // dQ kernel: 512 rows per block
+    int dq_rows, dq_qtiles, dq_slots;
+    long long dq_blocks;
+};
+BwdPlan plan_bwd(int D, bool f32, unsigned flags, int B, int Hq, int Hkv, int Sq, int q_split, const int *q_pos0, const ChunkDev *chunk,
+                 int n_chunks) {
+    BwdPlan pl;
+    if (f32) {
+        pl.wide_kv = pl.wide_q = false;
+        pl.keys_per_block = 64;
+        pl.kv_tiles = 0;
+        for (int c = 0; c < n_chunks; c++) pl.kv_tiles += (chunk[c].sk + 63) / 64;
+        pl.kv_blocks = pl.kv_tiles * B * Hkv;
+        pl.dq_rows = 64;
+        pl.dq_qtiles = pl.dq_slots = (Sq + 63) / 64;
+        pl.dq_blocks = (long long)pl.dq_qtiles * B * Hq;
+        return pl;
+    }
+    const bool causal_ = (flags & LTR_CAUSAL) != 0;
+    // keys per block of the dK/dV kernel: 256 (two 32-key halves per wave, about 12 % less time per key) pays at head dim 64
+    // when the wider blocks fill the device's CUs about as evenly as the 128-key blocks do (equal blocks, no mask), or, under
+    // a causal mask (unequal blocks), when a block walks many q tiles and there are several rounds of blocks to balance
+    // with; the caller can force either size
+    bool wide = (flags & LTR_DKDV_KEYS_256) != 0;
+    if (!wide && !(flags & LTR_DKDV_KEYS_128) && D == 64 && !(flags & LTR_NO_DKDV)) {
+        long long blocks256 = 0, blocks128 = 0;
+        for (int c = 0; c < n_chunks; c++) {
+            blocks256 += (chunk[c].sk + 255) / 256;
+            blocks128 += (chunk[c].sk + 127) / 128;
+        }
+        blocks256 *= (long long)B * Hkv;
+        blocks128 *= (long long)B * Hkv;
+        const long long q_tiles = (long long)(Hq / Hkv) * ((Sq + 63) / 64);
+        const int cus = device_cus();
+        if (causal_) wide = q_tiles >= 96 && blocks256 >= 4LL * cus;
+        else wide = q_tiles >= 16 && cu_fill(blocks256, cus) * 1.12 >= cu_fill(blocks128, cus);
+    }
+    pl.wide_kv = wide;
+    pl.keys_per_block = wide ? BwdLds<64, 2>::BN : BwdLds<64, 1>::BN;
+    pl.kv_tiles = 0;
+    for (int c = 0; c < n_chunks; c++) pl.kv_tiles += (chunk[c].sk + pl.keys_per_block - 1) / pl.keys_per_block;
+    pl.kv_blocks = pl.kv_tiles * B * Hkv;
+    // query rows per block of the dQ kernel: 512 (two 32-row blocks per wave) pays at head dim 64 when the wider blocks still
+    // fill the device, and under a causal mask only on sequences long enough that the diagonal does not dominate
+    bool wide_q = (flags & LTR_DQ_ROWS_512) != 0;
+    if (!wide_q && !(flags & LTR_DQ_ROWS_256) && D == 64 && !(flags & LTR_NO_DQ)) {
+        const int tiles512 = (Sq + 511) / 512;
+        const int slots512 = q_tile_slots(tiles512, (long long)B * Hq, causal_ && q_tiles_uneven(Sq, 512, q_split, q_pos0, chunk, n_chunks));
+        const long long blocks512 = (long long)slots512 * B * Hq;
+        const int cus = device_cus();
+        // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance; no mask: the wider
+        // blocks (about 7 % less time per row) must fill the CUs about as evenly as the 256-row blocks
+        const long long blocks256 = (long long)((Sq + 255) / 256) * B * Hq;
+        wide_q = causal_ ? (Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus)
+                         : (cu_fill(blocks512, cus) * 1.07 >= cu_fill(blocks256, cus));
+    }
+    pl.wide_q = wide_q;
+    pl.dq_rows = wide_q ? 512 : 256;
+    pl.dq_qtiles = (Sq + pl.dq_rows - 1) / pl.dq_rows;
+    pl.dq_slots = q_tile_slots(pl.dq_qtiles, (long long)B * Hq, causal_ && q_tiles_uneven(Sq, pl.dq_rows, q_split, q_pos0, chunk, n_chunks));
+    pl.dq_blocks = (long long)pl.dq_slots * B * Hq;
+    return pl;
 }
 
 // every position of the local rows lies inside the rows [pos0, pos0 + len) of a RoPE table
@@ -2357,39 +2484,19 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     p.n_chunks = a->n_chunks;
     hipStream_t st = (hipStream_t)stream;
     if ((a->flags & LTR_FWD_ROWS_512) && (a->D != 64 || a->io_dtype != LTR_BF16)) return LTR_EUNSUP;
+    const FwdPlan pl = plan_fwd(a->D, a->io_dtype == LTR_F32, a->flags, p.B, p.Hq, p.Sq, p.q_split, p.q_pos0, p.chunk, p.n_chunks);
+    if (pl.blocks > 0x7fffffffLL) return LTR_EINVAL;
+    p.n_qtiles = pl.n_qtiles;
+    p.n_slots = pl.n_slots;
     if (a->io_dtype == LTR_BF16) {
-        if ((long long)((p.Sq + 255) / 256) * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
-        const bool causal_ = (p.flags & LTR_CAUSAL) != 0;
-        // query rows per block: 512 (two 32-row blocks per wave, 64-key tiles) pays at head dim 64 under the conditions of
-        // the dQ kernel's 512-row blocks (see bwd_launch)
-        bool wide = (a->flags & LTR_FWD_ROWS_512) != 0;
-        if (!wide && !(a->flags & LTR_FWD_ROWS_256) && a->D == 64) {
-            const int tiles512 = (p.Sq + 511) / 512;
-            const int slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_ && q_tiles_uneven(p.Sq, 512, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
-            const long long blocks512 = (long long)slots512 * p.B * p.Hq, blocks256 = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
-            const int cus = device_cus();
-            wide = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus)
-                           : (cu_fill(blocks512, cus) * 1.07 >= cu_fill(blocks256, cus));
-        }
-        const int rows = wide ? 512 : 256;
-        p.n_qtiles = (p.Sq + rows - 1) / rows;
-        p.n_slots = q_tile_slots(p.n_qtiles, (long long)p.B * p.Hq,
-                                 causal_ && q_tiles_uneven(p.Sq, rows, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
-        const long long nblk = (long long)p.n_slots * p.B * p.Hq;
         rc = enable_large_lds();
         if (rc) return rc;
-        if (a->D == 128) hipLaunchKernelGGL((fwd_bf16_kernel<128, 1>), dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<128>(), st, p);
-        else if (wide) hipLaunchKernelGGL((fwd_bf16_kernel<64, 2>), dim3((unsigned)nblk), dim3(512), (fwd_lds_bytes<64, 2>()), st, p);
-        else hipLaunchKernelGGL((fwd_bf16_kernel<64, 1>), dim3((unsigned)nblk), dim3(512), fwd_lds_bytes<64>(), st, p);
-    } else {
-        p.n_qtiles = (p.Sq + 63) / 64;
-        p.n_slots = p.n_qtiles;
-        const long long nblk = (long long)p.n_qtiles * p.B * p.Hq;
-        if (nblk > 0x7fffffffLL) return LTR_EINVAL;
-        if (a->D == 128) hipLaunchKernelGGL(fwd_f32_kernel<128>, dim3((unsigned)nblk), dim3(64), 0, st, p);
-        else hipLaunchKernelGGL(fwd_f32_kernel<64>, dim3((unsigned)nblk), dim3(64), 0, st, p);
+        if (a->D == 128) return launch((const void *)fwd_bf16_kernel<128, 1>, pl.blocks, 512, fwd_lds_bytes<128>(), st, p);
+        if (pl.wide) return launch((const void *)fwd_bf16_kernel<64, 2>, pl.blocks, 512, fwd_lds_bytes<64, 2>(), st, p);
+        return launch((const void *)fwd_bf16_kernel<64, 1>, pl.blocks, 512, fwd_lds_bytes<64>(), st, p);
     }
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    if (a->D == 128) return launch((const void *)fwd_f32_kernel<128>, pl.blocks, 64, 0, st, p);
+    return launch((const void *)fwd_f32_kernel<64>, pl.blocks, 64, 0, st, p);
 }
 
 extern "C" int ltr_attn_bwd_delta(const ltr_attn_delta_args *a, void *stream) {
@@ -2419,8 +2526,7 @@ extern "C" int ltr_attn_bwd_delta(const ltr_attn_delta_args *a, void *stream) {
     const long long nthreads = (long long)p.B * p.Hq * p.Sq * 16;
     const long long nblk = (nthreads + 255) / 256;
     if (nblk > 0x7fffffffLL) return LTR_EINVAL;
-    hipLaunchKernelGGL(delta_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream, p);
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    return launch((const void *)delta_kernel, nblk, 256, 0, (hipStream_t)stream, p);
 }
 
 namespace {
@@ -2470,29 +2576,8 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         p.rope = a->rope_freqs;
         p.rope_pos0 = (int)a->rope_pos0;
     }
-    // keys per block of the dK/dV kernel: 256 (two 32-key halves per wave, about 12 % less time per key) pays at head dim 64
-    // when the wider blocks fill the device's CUs about as evenly as the 128-key blocks do (equal blocks, no mask), or, under
-    // a causal mask (unequal blocks), when a block walks many q tiles and there are several rounds of blocks to balance
-    // with; the caller can force either size
-    bool wide = false;
-    if (flags & LTR_DKDV_KEYS_256) {
-        if (a->D != 64 || f32) return LTR_EUNSUP;
-        wide = true;
-    } else if (!(flags & LTR_DKDV_KEYS_128) && a->D == 64 && !f32 && do_dkdv) {
-        long long blocks256 = 0, blocks128 = 0;
-        for (int c = 0; c < a->n_chunks; c++) {
-            blocks256 += (a->chunk[c].sk + 255) / 256;
-            blocks128 += (a->chunk[c].sk + 127) / 128;
-        }
-        blocks256 *= (long long)a->B * a->Hkv;
-        blocks128 *= (long long)a->B * a->Hkv;
-        const long long q_tiles = (long long)(a->Hq / a->Hkv) * ((a->Sq + 63) / 64);
-        const int cus = device_cus();
-        if (flags & LTR_CAUSAL) wide = q_tiles >= 96 && blocks256 >= 4LL * cus;
-        else wide = q_tiles >= 16 && cu_fill(blocks256, cus) * 1.12 >= cu_fill(blocks128, cus);
-    }
-    const int keys_per_block = wide ? BwdLds<64, 2>::BN : BwdLds<64, 1>::BN;
-    long long tiles = 0;
+    if ((flags & LTR_DKDV_KEYS_256) && (a->D != 64 || f32)) return LTR_EUNSUP;
+    if ((flags & LTR_DQ_ROWS_512) && a->D != 64) return LTR_EUNSUP;
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];
         if (!ch.k || !ch.v || ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
@@ -2506,7 +2591,6 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         p.chunk[c].dv = (float *)ch.dv;
         p.chunk[c].sk = (int)ch.sk;
         p.chunk[c].pos0 = (int)ch.pos0;
-        tiles += (ch.sk + keys_per_block - 1) / keys_per_block;
     }
     int rc = check_device();
     if (rc) return rc;
@@ -2542,60 +2626,34 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     p.scale = a->scale;
     p.flags = flags;
     p.n_chunks = a->n_chunks;
-    p.tiles_total = (int)tiles;
-    const long long nblk = tiles * p.B * p.Hkv;
-    if (nblk > 0x7fffffffLL) return LTR_EINVAL;
+    const BwdPlan pl = plan_bwd(a->D, f32, flags, p.B, p.Hq, p.Hkv, p.Sq, p.q_split, p.q_pos0, p.chunk, p.n_chunks);
+    if (pl.kv_blocks > 0x7fffffffLL || pl.dq_blocks > 0x7fffffffLL) return LTR_EINVAL;
+    p.tiles_total = (int)pl.kv_tiles;
+    p.n_slots = pl.dq_slots;
     hipStream_t st = (hipStream_t)stream;
     if (f32) {
-        long long tiles64 = 0;
-        for (int c = 0; c < a->n_chunks; c++) tiles64 += (a->chunk[c].sk + 63) / 64;
-        const long long nq = (long long)((p.Sq + 63) / 64) * p.B * p.Hq, nk = tiles64 * p.B * p.Hkv;
-        if (nq > 0x7fffffffLL || nk > 0x7fffffffLL) return LTR_EINVAL;
-        if (a->D == 128) {
-            if (do_dq) hipLaunchKernelGGL(bwd_dq_f32_kernel<128>, dim3((unsigned)nq), dim3(64), 0, st, p);
-            if (do_dkdv) {
-                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<128, false>), dim3((unsigned)nk), dim3(64), 0, st, p);
-                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<128, true>), dim3((unsigned)nk), dim3(64), 0, st, p);
-            }
-        } else {
-            if (do_dq) hipLaunchKernelGGL(bwd_dq_f32_kernel<64>, dim3((unsigned)nq), dim3(64), 0, st, p);
-            if (do_dkdv) {
-                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<64, false>), dim3((unsigned)nk), dim3(64), 0, st, p);
-                hipLaunchKernelGGL((bwd_dkdv_f32_kernel<64, true>), dim3((unsigned)nk), dim3(64), 0, st, p);
-            }
+        if (do_dq) {
+            rc = a->D == 128 ? launch((const void *)bwd_dq_f32_kernel<128>, pl.dq_blocks, 64, 0, st, p)
+                             : launch((const void *)bwd_dq_f32_kernel<64>, pl.dq_blocks, 64, 0, st, p);
+            if (rc) return rc;
         }
-        return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+        if (do_dkdv) {
+            rc = a->D == 128 ? launch((const void *)bwd_dkdv_f32_kernel<128, false>, pl.kv_blocks, 64, 0, st, p)
+                             : launch((const void *)bwd_dkdv_f32_kernel<64, false>, pl.kv_blocks, 64, 0, st, p);
+            if (rc) return rc;
+            rc = a->D == 128 ? launch((const void *)bwd_dkdv_f32_kernel<128, true>, pl.kv_blocks, 64, 0, st, p)
+                             : launch((const void *)bwd_dkdv_f32_kernel<64, true>, pl.kv_blocks, 64, 0, st, p);
+        }
+        return rc;
     }
     rc = enable_large_lds();
     if (rc) return rc;
-    if ((long long)((p.Sq + 255) / 256) * p.B * p.Hq > 0x7fffffffLL) return LTR_EINVAL;
-    // query rows per block of the dQ kernel: 512 (two 32-row blocks per wave) pays at head dim 64 when the wider blocks still
-    // fill the device, and under a causal mask only on sequences long enough that the diagonal does not dominate
-    bool wide_q = false;
-    if (flags & LTR_DQ_ROWS_512) {
-        if (a->D != 64) return LTR_EUNSUP;
-        wide_q = true;
-    } else if (!(flags & LTR_DQ_ROWS_256) && a->D == 64 && do_dq) {
-        const bool causal_ = (flags & LTR_CAUSAL) != 0;
-        const int tiles512 = (p.Sq + 511) / 512;
-        const int slots512 = q_tile_slots(tiles512, (long long)p.B * p.Hq, causal_ && q_tiles_uneven(p.Sq, 512, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
-        const long long blocks512 = (long long)slots512 * p.B * p.Hq;
-        const int cus = device_cus();
-        // causal: equal (paired) blocks need one full round, unequal ones several rounds to balance; no mask: the wider
-        // blocks (about 7 % less time per row) must fill the CUs about as evenly as the 256-row blocks
-        const long long blocks256 = (long long)((p.Sq + 255) / 256) * p.B * p.Hq;
-        wide_q = causal_ ? (p.Sq >= 2048 && blocks512 >= (long long)(slots512 != tiles512 ? 1 : 4) * cus)
-                         : (cu_fill(blocks512, cus) * 1.07 >= cu_fill(blocks256, cus));
-    }
-    const int dq_rows = wide_q ? 512 : 256;
-    p.n_slots = q_tile_slots((p.Sq + dq_rows - 1) / dq_rows, (long long)p.B * p.Hq,
-                             (flags & LTR_CAUSAL) && q_tiles_uneven(p.Sq, dq_rows, p.q_split, p.q_pos0, p.chunk, p.n_chunks));
-    const long long nblk_q = (long long)p.n_slots * p.B * p.Hq;
     // the dQ kernel goes first: with LTR_DELTA_FROM_O it produces the DELTA that the dK/dV kernel reads
     if (do_dq) {
-        if (a->D == 128) hipLaunchKernelGGL((bwd_dq_kernel<128, 1>), dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<128>(), st, p);
-        else if (wide_q) hipLaunchKernelGGL((bwd_dq_kernel<64, 2>), dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
-        else hipLaunchKernelGGL((bwd_dq_kernel<64, 1>), dim3((unsigned)nblk_q), dim3(512), dq_lds_bytes<64>(), st, p);
+        if (a->D == 128) rc = launch((const void *)bwd_dq_kernel<128, 1>, pl.dq_blocks, 512, dq_lds_bytes<128>(), st, p);
+        else if (pl.wide_q) rc = launch((const void *)bwd_dq_kernel<64, 2>, pl.dq_blocks, 512, dq_lds_bytes<64>(), st, p);
+        else rc = launch((const void *)bwd_dq_kernel<64, 1>, pl.dq_blocks, 512, dq_lds_bytes<64>(), st, p);
+        if (rc) return rc;
     }
     if (do_dkdv) {
         // A block of the dK/dV kernel owns 128 keys and loops over the query tiles that see them: under a causal mask its
@@ -2604,17 +2662,65 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
         // the tail (the sums inside a block do not depend on the table's order).
         if (flags & LTR_CAUSAL)
             std::stable_sort(p.chunk, p.chunk + p.n_chunks, [](const ChunkDev &x, const ChunkDev &y) { return x.pos0 < y.pos0; });
-        if (a->D == 128) hipLaunchKernelGGL((bwd_dkdv_kernel<128, 1>), dim3((unsigned)nblk), dim3(BwdLds<128, 1>::NT), (BwdLds<128, 1>::TOTAL), st, p);
-        else if (wide) hipLaunchKernelGGL((bwd_dkdv_kernel<64, 2>), dim3((unsigned)nblk), dim3(BwdLds<64, 2>::NT), (BwdLds<64, 2>::TOTAL), st, p);
-        else hipLaunchKernelGGL((bwd_dkdv_kernel<64, 1>), dim3((unsigned)nblk), dim3(BwdLds<64, 1>::NT), (BwdLds<64, 1>::TOTAL), st, p);
+        if (a->D == 128) rc = launch((const void *)bwd_dkdv_kernel<128, 1>, pl.kv_blocks, BwdLds<128, 1>::NT, BwdLds<128, 1>::TOTAL, st, p);
+        else if (pl.wide_kv) rc = launch((const void *)bwd_dkdv_kernel<64, 2>, pl.kv_blocks, BwdLds<64, 2>::NT, BwdLds<64, 2>::TOTAL, st, p);
+        else rc = launch((const void *)bwd_dkdv_kernel<64, 1>, pl.kv_blocks, BwdLds<64, 1>::NT, BwdLds<64, 1>::TOTAL, st, p);
     }
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    return rc;
 }
 }  // namespace
 
 extern "C" int ltr_attn_bwd(const ltr_attn_bwd_args *a, void *stream) {
     if (!a) return LTR_EINVAL;
     return bwd_launch(a, a->flags, false, stream);
+}
+
+// Host-only: nothing is enqueued, no pointer is read.
+extern "C" int ltr_attn_plan(const ltr_attn_bwd_args *a, ltr_attn_plan_t *out) {
+    if (!a || !out) return LTR_EINVAL;
+    if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
+    if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
+    if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
+    if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
+    if (!fits_i32(a->Sq) || a->q_split < 0 || a->q_split > a->Sq) return LTR_EINVAL;
+    if (!fits_i32(a->q_pos0[0] + a->Sq) || !fits_i32(a->q_pos0[1] + a->Sq)) return LTR_EINVAL;
+    const unsigned flags = a->flags;
+    if ((flags & LTR_DKDV_KEYS_128) && (flags & LTR_DKDV_KEYS_256)) return LTR_EINVAL;
+    if ((flags & LTR_DQ_ROWS_256) && (flags & LTR_DQ_ROWS_512)) return LTR_EINVAL;
+    if ((flags & LTR_FWD_ROWS_256) && (flags & LTR_FWD_ROWS_512)) return LTR_EINVAL;
+    const bool f32 = a->io_dtype == LTR_F32;
+    if ((flags & (LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_512 | LTR_FWD_ROWS_512)) && (a->D != 64 || f32)) return LTR_EUNSUP;
+    ChunkDev chunk[LTR_MAX_CHUNKS];
+    for (int c = 0; c < a->n_chunks; c++) {
+        const ltr_kv_chunk &ch = a->chunk[c];
+        if (ch.sk <= 0 || !fits_i32(ch.sk) || !fits_i32(ch.pos0 + ch.sk)) return LTR_EINVAL;
+        chunk[c].k = chunk[c].v = nullptr;
+        chunk[c].dk = chunk[c].dv = nullptr;
+        chunk[c].sk = (int)ch.sk;
+        chunk[c].pos0 = (int)ch.pos0;
+    }
+    const int q_pos0[2] = {(int)a->q_pos0[0], (int)a->q_pos0[1]};
+    const FwdPlan f = plan_fwd(a->D, f32, flags, a->B, a->Hq, (int)a->Sq, (int)a->q_split, q_pos0, chunk, a->n_chunks);
+    const BwdPlan b = plan_bwd(a->D, f32, flags, a->B, a->Hq, a->Hkv, (int)a->Sq, (int)a->q_split, q_pos0, chunk, a->n_chunks);
+    out->compute_units = device_cus();
+    out->fwd_rows = f.rows;
+    out->fwd_paired = f.n_slots != f.n_qtiles;
+    out->fwd_blocks = f.blocks;
+    out->dq_rows = b.dq_rows;
+    out->dq_paired = b.dq_slots != b.dq_qtiles;
+    out->dq_blocks = b.dq_blocks;
+    out->dkdv_keys = b.keys_per_block;
+    out->dkdv_blocks = b.kv_blocks;
+    if (f32) {
+        snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_f32_kernel<%d>", a->D);
+        snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_f32_kernel<%d>", a->D);
+        snprintf(out->dkdv_kernel, sizeof(out->dkdv_kernel), "bwd_dkdv_f32_kernel<%d, *>", a->D);
+    } else {
+        snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_bf16_kernel<%d, %d>", a->D, f.wide ? 2 : 1);
+        snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_kernel<%d, %d>", a->D, b.wide_q ? 2 : 1);
+        snprintf(out->dkdv_kernel, sizeof(out->dkdv_kernel), "bwd_dkdv_kernel<%d, %d>", a->D, b.wide_kv ? 2 : 1);
+    }
+    return LTR_OK;
 }
 
 extern "C" int ltr_attn_bwd_noalloc(const ltr_attn_bwd_args *a, void *stream) {
@@ -2636,7 +2742,10 @@ extern "C" int ltr_cast_f32_to_bf16(const float *src, void *dst, int64_t n, void
     if (rc) return rc;
     const long long nblk = (n / 4 + 256) / 256;
     if (nblk > 0x7fffffffLL) return LTR_EINVAL;
-    hipLaunchKernelGGL(cast_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream, src, (__bf16 *)dst,
-                       (long long)n);
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    __bf16 *dst16 = (__bf16 *)dst;
+    long long n64 = n;
+    void *args[] = {(void *)&src, (void *)&dst16, (void *)&n64};
+    return hipLaunchKernel((const void *)cast_kernel, dim3((unsigned)nblk), dim3(256), args, 0, (hipStream_t)stream) == hipSuccess
+               ? LTR_OK
+               : LTR_ELAUNCH;
 }

@@ -1,5 +1,6 @@
-// Measurement helpers of the attention library (gfx950): what this device sustains on the matrix pipe, and at which
-// shader clock, so that a benchmark can print the kernels' rates beside the device's own ceiling.
+// Measurement helpers for benchmarks of the attention library (gfx950), built into a library of their own
+// (libltr_probe.so, include/ltr_probe.h): what this device sustains on the matrix pipe, and at which shader clock, so
+// that a benchmark can print the kernels' rates beside the device's own ceiling.  Nothing here is on the attention path.
 //   mfma_probe_kernel   every wave runs four independent accumulation chains of v_mfma_f32_32x32x16_bf16 on operands that
 //                       stay in registers (no memory traffic inside the loop): the matrix pipe is the only limit.  With
 //                       operands taken from the caller's workspace (random data) the chip runs at the clock its power
@@ -8,7 +9,7 @@
 //   loop (their ratio is the shader clock under this load); the rate is taken by the caller over the whole launch.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include "ltr_attn.h"
+#include "ltr_probe.h"
 
 namespace {
 
@@ -56,58 +57,13 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(const uint4 *operands, 
     }
 }
 
-// What a fused backward (dQ produced by the blocks that own keys) would have to do once per 64-row step: add a 64 x 128
-// fp32 partial dQ tile into memory that the blocks of other key ranges add to as well.  Eight waves, each adding one
-// 32 x 32 tile in MFMA accumulator layout (a half-wave = 128 contiguous bytes of one row), to the rows of (head, q tile)
-// = the step's place in a walk over `heads` x 64 tiles; blocks of one XCD (block index mod 8) walk the same heads, each
-// starting at its own tile, like key blocks of one kv head would.  with_mfma: 40 MFMAs per wave between two tile adds
-// (the matrix work of such a step), to see whether the adds hide under it.
-__global__ __launch_bounds__(512) void atomic_tile_add_kernel(float *dq, const uint4 *operands, int n_operands, int steps, int with_mfma,
-                                                              float *sink) {
-    extern __shared__ unsigned char probe_lds[];   // sized by the launch so that one block fits a CU
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, l32 = lane & 31, hh = lane >> 5;
-    const int grp = blockIdx.x & 7, j = blockIdx.x >> 3;
-    union { uint4 u; bf16x8 v; } a, b;
-    a.u = operands[(2 * tid) % n_operands];
-    b.u = operands[(2 * tid + 1) % n_operands];
-    f32x16 c0, c1, c2, c3;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        c0[r] = 0.f;
-        c1[r] = 1.f;
-        c2[r] = 2.f;
-        c3[r] = 3.f;
-    }
-    for (int s = 0; s < steps; s++) {
-        const int h = grp * 4 + ((s >> 6) & 3), qt = (s + 2 * j) & 63;
-        if (with_mfma) {
-            for (int it = 0; it < 10; it++) {
-                c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c0, 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c1, 0, 0, 0);
-                c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c2, 0, 0, 0);
-                c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c3, 0, 0, 0);
-            }
-        }
-        float *base = dq + ((long long)(h * 4096 + qt * 64)) * 128;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int row = 32 * (w >> 2) + 8 * (r >> 2) + 4 * hh + (r & 3), col = 32 * (w & 3) + l32;
-            unsafeAtomicAdd(base + row * 128 + col, 1.0f);   // the hardware's fp32 add (global_atomic_add_f32), no CAS loop
-        }
-    }
-    float sum = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) sum += c0[r] + c1[r] + c2[r] + c3[r];
-    if (sum == 12345.678f) sink[tid & 1023] = sum;
-}
-
 }  // namespace
 
 extern "C" int ltr_device_info(ltr_device_info_t *out) {
-    if (!out) return LTR_EINVAL;
+    if (!out) return LTR_PROBE_EINVAL;
     int dev = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_EDEVICE;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_PROBE_EDEVICE;
     out->compute_units = prop.multiProcessorCount;
     out->clock_khz = prop.clockRate;
     out->memory_clock_khz = prop.memoryClockRate;
@@ -117,47 +73,28 @@ extern "C" int ltr_device_info(ltr_device_info_t *out) {
     int i = 0;
     for (; i < 63 && prop.gcnArchName[i]; i++) out->arch[i] = prop.gcnArchName[i];
     out->arch[i] = 0;
-    return LTR_OK;
+    return LTR_PROBE_OK;
 }
 
 extern "C" int ltr_probe_mfma(void *workspace, int64_t workspace_bytes, int32_t iters, int32_t random_operands, void *stream) {
-    if (!workspace || iters <= 0) return LTR_EINVAL;
-    if (workspace_bytes < LTR_PROBE_MIN_WORKSPACE) return LTR_EINVAL;
-    if ((uintptr_t)workspace & 15) return LTR_EALIGN;
+    if (!workspace || iters <= 0) return LTR_PROBE_EINVAL;
+    if (workspace_bytes < LTR_PROBE_MIN_WORKSPACE) return LTR_PROBE_EINVAL;
+    if ((uintptr_t)workspace & 15) return LTR_PROBE_EALIGN;
     int dev = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_EDEVICE;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_PROBE_EDEVICE;
     const char *a = prop.gcnArchName;
-    if (!(a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')) return LTR_EDEVICE;
+    if (!(a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')) return LTR_PROBE_EDEVICE;
     // layout of the workspace: [0, 16) two tick counts (results), [4096, 8192) sink, [8192, ...) operands (read only)
     long long *ticks = (long long *)workspace;
     float *sink = (float *)((char *)workspace + 4096);
     const uint4 *operands = (const uint4 *)((char *)workspace + 8192);
-    const int n_operands = (int)((workspace_bytes - 8192) / 16);
-    hipLaunchKernelGGL(mfma_probe_kernel, dim3(prop.multiProcessorCount), dim3(512), 0, (hipStream_t)stream, operands, n_operands,
-                       iters, random_operands, sink, ticks);
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    int n_operands = (int)((workspace_bytes - 8192) / 16);
+    int iters_ = iters, random_ = random_operands;
+    void *args[] = {(void *)&operands, (void *)&n_operands, (void *)&iters_, (void *)&random_, (void *)&sink, (void *)&ticks};
+    return hipLaunchKernel((const void *)mfma_probe_kernel, dim3(prop.multiProcessorCount), dim3(512), args, 0, (hipStream_t)stream) ==
+                   hipSuccess
+               ? LTR_PROBE_OK
+               : LTR_PROBE_ELAUNCH;
 }
 
-extern "C" int ltr_probe_atomic_tile_add(float *dst, int64_t dst_elems, void *workspace, int64_t workspace_bytes, int32_t steps,
-                                         int32_t with_mfma, void *stream) {
-    if (!dst || !workspace || steps <= 0) return LTR_EINVAL;
-    if (dst_elems < (int64_t)32 * 4096 * 128 || workspace_bytes < LTR_PROBE_MIN_WORKSPACE) return LTR_EINVAL;
-    if (((uintptr_t)dst | (uintptr_t)workspace) & 15) return LTR_EALIGN;
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return LTR_EDEVICE;
-    const char *a = prop.gcnArchName;
-    if (!(a[0] == 'g' && a[1] == 'f' && a[2] == 'x' && a[3] == '9' && a[4] == '5' && a[5] == '0')) return LTR_EDEVICE;
-    constexpr int LDS = 96 * 1024;   // more than half a CU's LDS: one block per CU, like the attention kernels
-    if (hipFuncSetAttribute((const void *)atomic_tile_add_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
-        (void)hipGetLastError();
-        return LTR_ELAUNCH;
-    }
-    float *sink = (float *)((char *)workspace + 4096);
-    const uint4 *operands = (const uint4 *)((char *)workspace + 8192);
-    const int n_operands = (int)((workspace_bytes - 8192) / 16);
-    hipLaunchKernelGGL(atomic_tile_add_kernel, dim3(256), dim3(512), LDS, (hipStream_t)stream, dst, operands, n_operands, steps,
-                       with_mfma, sink);
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
-}

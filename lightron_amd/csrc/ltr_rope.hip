@@ -134,12 +134,10 @@ extern "C" int ltr_rope_apply(const ltr_rope_args *a, void *stream) {
     const unsigned grid = (unsigned)((n_units + 255) / 256);
     const bool small = n_units + 256 < 0xffffffffLL;
     hipStream_t st = (hipStream_t)stream;
-    if (a->io_dtype == LTR_BF16) {
-        if (small) hipLaunchKernelGGL((rope_kernel<true, unsigned>), dim3(grid), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((rope_kernel<true, unsigned long long>), dim3(grid), dim3(256), 0, st, p);
-    } else {
-        if (small) hipLaunchKernelGGL((rope_kernel<false, unsigned>), dim3(grid), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL((rope_kernel<false, unsigned long long>), dim3(grid), dim3(256), 0, st, p);
-    }
-    return hipGetLastError() == hipSuccess ? LTR_OK : LTR_ELAUNCH;
+    // the launch's own status (an error left behind by unrelated earlier work is neither reported as ours nor cleared)
+    const void *kernel = a->io_dtype == LTR_BF16
+                             ? (small ? (const void *)rope_kernel<true, unsigned> : (const void *)rope_kernel<true, unsigned long long>)
+                             : (small ? (const void *)rope_kernel<false, unsigned> : (const void *)rope_kernel<false, unsigned long long>);
+    void *args[] = {(void *)&p};
+    return hipLaunchKernel(kernel, dim3(grid), dim3(256), args, 0, st) == hipSuccess ? LTR_OK : LTR_ELAUNCH;
 }

@@ -21,15 +21,38 @@ def _lib():
     return L, L.load()
 
 
+def _declared(header):
+    hdr = open(os.path.join(ROOT, "include", header)).read()
+    return set(re.findall(r"^(?:int|const char \*)\s*\*?(ltr_\w+)\(", hdr, flags=re.M))
+
+
+def _exported(path):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    return {ln.split()[-1] for ln in out.splitlines() if " T " in ln and ln.split()[-1].startswith("ltr_")}
+
+
 def test_header_symbols_exported():
     L, lib = _lib()
-    hdr = open(os.path.join(ROOT, "include", "ltr_attn.h")).read()
-    declared = set(re.findall(r"^(?:int|const char \*)\s*\*?(ltr_\w+)\(", hdr, flags=re.M))
+    declared = _declared("ltr_attn.h")
     assert declared == set(L.EXPORTS), declared
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.ltr_abi_version() == 7
+    # the product library exports the attention path and nothing else
+    assert _exported(L.LIB_PATH) == declared
+    assert lib.ltr_abi_version() == 8
     assert lib.ltr_strerror(0) == b"ok" and b"aligned" in lib.ltr_strerror(-3)
+
+
+def test_probe_library_is_separate():
+    """The measurement helpers of bench.py live in a library of their own (include/ltr_probe.h)."""
+    L, _ = _lib()
+    probe = L.load_probe()
+    declared = _declared("ltr_probe.h")
+    assert declared == set(L.PROBE_EXPORTS) == _exported(L.PROBE_LIB_PATH)
+    for name in declared:
+        assert getattr(probe, name) is not None
+    assert probe.ltr_device_info(None) == -1 and probe.ltr_probe_mfma(None, 0, 1, 0, None) == -1
 
 
 def test_struct_layout_matches_header():
@@ -40,6 +63,54 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(L.DeltaArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
     assert ctypes.sizeof(L.BwdArgs) == 5 * 8 + 4 * 4 + 8 + 7 * 24 + 16 + 8 + 4 * 4 + 32 * 48 + 8 + 24 + 3 * 8
     assert ctypes.sizeof(L.RopeArgs) == 3 * 8 + 3 * 4 + 4 + 8 + 2 * 24 + 2 * 4
+    assert ctypes.sizeof(L.DeviceInfo) == 4 * 4 + 2 * 8 + 64
+
+
+def _plan(L, lib, D, B, Hq, Hkv, Sq, chunks, flags=0, dtype=None, q_pos0=(0, 0), q_split=None):
+    a = L.BwdArgs()
+    a.B, a.Hq, a.Hkv, a.D, a.Sq, a.n_chunks = B, Hq, Hkv, D, Sq, len(chunks)
+    a.q_pos0[0], a.q_pos0[1], a.q_split = q_pos0[0], q_pos0[1], Sq if q_split is None else q_split
+    a.flags, a.io_dtype = flags, L.LTR_BF16 if dtype is None else dtype
+    for i, (sk, pos0) in enumerate(chunks):
+        a.chunk[i].sk, a.chunk[i].pos0 = sk, pos0
+    out = L.AttnPlan()
+    rc = lib.ltr_attn_plan(ctypes.byref(a), ctypes.byref(out))
+    return rc, out
+
+
+def test_plan_names_the_kernels_and_follows_the_hints():
+    """ltr_attn_plan (host only; 256 compute units without a device) answers with the block sizes the launches would use:
+    head dim 128 has one size of each kernel, head dim 64 two, and every LTR_*_ROWS_* / LTR_DKDV_KEYS_* hint forces its size."""
+    L, lib = _lib()
+    assert ctypes.sizeof(L.AttnPlan) == 6 * 4 + 3 * 8 + 3 * 48
+    assert lib.ltr_attn_plan(None, None) == -1
+    # config 3, one zig-zag rank share: 16 half-chunks of 2048 keys
+    hc = 2048
+    rc, pl = _plan(L, lib, 128, 1, 32, 8, 4096, [(hc, i * hc) for i in range(16)], L.LTR_CAUSAL, q_pos0=(0, 15 * hc), q_split=hc)
+    assert rc == 0 and pl.compute_units > 0
+    assert (pl.fwd_kernel, pl.dq_kernel, pl.dkdv_kernel) == (b"fwd_bf16_kernel<128, 1>", b"bwd_dq_kernel<128, 1>", b"bwd_dkdv_kernel<128, 1>")
+    assert (pl.fwd_rows, pl.dq_rows, pl.dkdv_keys) == (256, 256, 128)
+    assert pl.dkdv_blocks == 16 * (hc // 128) * 8 and pl.fwd_blocks == pl.dq_blocks
+    assert pl.fwd_blocks in (16 * 32, 8 * 32)            # one tile per block, or late + early tile paired
+    # head dim 64: both sizes exist; the hints force them, whatever the library would have chosen
+    shape = (64, 8, 4, 4, 4096, [(4096, 0)])
+    for fl, field, want in ((L.LTR_FWD_ROWS_256, "fwd_rows", 256), (L.LTR_FWD_ROWS_512, "fwd_rows", 512),
+                            (L.LTR_DQ_ROWS_256, "dq_rows", 256), (L.LTR_DQ_ROWS_512, "dq_rows", 512),
+                            (L.LTR_DKDV_KEYS_128, "dkdv_keys", 128), (L.LTR_DKDV_KEYS_256, "dkdv_keys", 256)):
+        rc, pl = _plan(L, lib, *shape, flags=fl)
+        assert rc == 0 and getattr(pl, field) == want, (fl, field)
+    rc, pl = _plan(L, lib, *shape, flags=L.LTR_DKDV_KEYS_256 | L.LTR_DQ_ROWS_512 | L.LTR_FWD_ROWS_512)
+    assert (pl.fwd_kernel, pl.dq_kernel, pl.dkdv_kernel) == (b"fwd_bf16_kernel<64, 2>", b"bwd_dq_kernel<64, 2>", b"bwd_dkdv_kernel<64, 2>")
+    assert pl.dkdv_blocks == (4096 // 256) * 8 * 4 and pl.fwd_blocks == (4096 // 512) * 8 * 4
+    rc, pl = _plan(L, lib, *shape)                         # config 5's shape: the library's own choice on 256 CUs
+    assert rc == 0 and pl.dkdv_keys in (128, 256) and pl.dkdv_blocks == (4096 // pl.dkdv_keys) * 32
+    # the wide blocks are bf16, head dim 64 only
+    assert _plan(L, lib, 128, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_DKDV_KEYS_256)[0] == -2
+    assert _plan(L, lib, 64, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_DQ_ROWS_512, dtype=L.LTR_F32)[0] == -2
+    assert _plan(L, lib, 64, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_DQ_ROWS_512 | L.LTR_DQ_ROWS_256)[0] == -1
+    assert _plan(L, lib, 96, 1, 4, 4, 512, [(512, 0)])[0] == -2
+    rc, pl = _plan(L, lib, 64, 2, 8, 8, 1024, [(256, 0)] * 4, dtype=L.LTR_F32)    # config 1's shape, scalar fp32 kernels
+    assert rc == 0 and pl.fwd_kernel == b"fwd_f32_kernel<64>" and pl.fwd_rows == 64 and pl.dkdv_blocks == 4 * 4 * 16
 
 
 def test_validation_without_gpu():
