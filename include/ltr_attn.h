@@ -65,6 +65,9 @@ extern "C" {
 #define LTR_FWD_ROWS_512 16384u /* forward, tuning hint: they own 512 rows (bf16, head dim 64 only: LTR_EUNSUP otherwise); results differ
                                    only through the tile size (64 instead of 128 keys: the order of fp32 additions) */
 
+#define LTR_FWD_F32_SCALAR 32768u /* forward, fp32 only: run the scalar fp32 kernel instead of the matrix-pipe one (same results to
+                                    rounding; the fallback and cross-check of fwd_f32_mfma_kernel) */
+
 /* error codes */
 #define LTR_OK 0
 #define LTR_EINVAL (-1)   /* null pointer, bad size, bad flag */
@@ -110,7 +113,7 @@ typedef struct ltr_attn_fwd_args {
     int64_t q_pos0[2];
     int64_t q_split;
     float scale;          /* 1/sqrt(D) at every reference call site (ring_attention.py:20) */
-    uint32_t flags;       /* LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q | LTR_FWD_ROWS_256 | LTR_FWD_ROWS_512 */
+    uint32_t flags;       /* LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q | LTR_FWD_ROWS_256 | LTR_FWD_ROWS_512 | LTR_FWD_F32_SCALAR */
     int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v */
     int32_t o_dtype;      /* LTR_BF16 or LTR_F32 */
     int32_t n_chunks;     /* 1..LTR_MAX_CHUNKS */
@@ -267,7 +270,7 @@ int ltr_rope_apply(const ltr_rope_args *args, void *stream);
  * for 256 compute units).  It has no counterpart in the reference (which leaves the choice of kernel to the library
  * behind F.scaled_dot_product_attention, model/model.py:193); it is for benchmarks and profiles that must name the kernel
  * they measured, and for tests of the size hints.  The sizes, strides' owner shapes, positions, chunk lengths, dtype and
- * flags of args are read; flags may also carry the forward's hints (LTR_FWD_ROWS_256 / LTR_FWD_ROWS_512).  The library's
+ * flags of args are read; flags may also carry the forward's hints (LTR_FWD_ROWS_256 / LTR_FWD_ROWS_512 / LTR_FWD_F32_SCALAR).  The library's
  * launches and this answer come from one function, so they cannot drift apart.  Kernel names are those a profiler shows.
  */
 typedef struct ltr_attn_plan_t {

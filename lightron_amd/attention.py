@@ -113,12 +113,14 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
              q_pos0=0, q_split: Optional[int] = None, causal: bool = False, scale: Optional[float] = None,
              out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None, merge: bool = False,
              out_dtype: Optional[torch.dtype] = None, q_rope: Optional[torch.Tensor] = None,
-             q_rot_out: Optional[torch.Tensor] = None, fwd_rows: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+             q_rot_out: Optional[torch.Tensor] = None, fwd_rows: Optional[int] = None,
+             f32_scalar: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """One Q chunk against a table of KV chunks -> (O [B,Sq,Hq,D], LSE [B,Hq,Sq] fp32).
     With merge=True, `out`/`lse` hold an earlier partial result which is merged in place.
     q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table whose row p belongs to global position p: q is un-rotated and the
     kernel's prologue applies RoPE to it (LTR_ROPE_Q; bf16 only); q_rot_out (bf16, like q) receives the rotated q.
-    fwd_rows: None (the library chooses), 256 or 512 query rows per block (512: bf16 with head dim 64 only)."""
+    fwd_rows: None (the library chooses), 256 or 512 query rows per block (512: bf16 with head dim 64 only).
+    f32_scalar: fp32 inputs only - the scalar fp32 kernel instead of the matrix-pipe one (LTR_FWD_F32_SCALAR)."""
     lib = _lib.load()
     _req(q, "q")
     B, Sq, Hq, D = q.shape
@@ -149,7 +151,7 @@ def attn_fwd(q: torch.Tensor, ks: Sequence[torch.Tensor], vs: Sequence[torch.Ten
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
     a.io_dtype, a.o_dtype = _DT[q.dtype], _DT[out.dtype]
-    rope_flag = 0
+    rope_flag = _lib.LTR_FWD_F32_SCALAR if f32_scalar else 0
     if fwd_rows is not None:
         if fwd_rows not in (256, 512):
             raise RuntimeError("fwd_rows must be None, 256 or 512")
@@ -301,7 +303,7 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
 
 def attn_plan(B: int, Hq: int, Hkv: int, D: int, Sq: int, chunk_lens: Sequence[int], k_pos0: Sequence[int], q_pos0=0,
               q_split: Optional[int] = None, causal: bool = False, dtype: torch.dtype = torch.bfloat16, fwd_rows=None,
-              dq_rows=None, dkdv_keys=None) -> dict:
+              dq_rows=None, dkdv_keys=None, f32_scalar: bool = False) -> dict:
     """Which kernels the library would launch for this problem on the current device (ltr_attn_plan: a host call, no
     tensors needed; at most 32 chunks = one launch): block sizes, block counts and the kernels' names as a profiler
     shows them.  fwd_rows / dq_rows / dkdv_keys force a size like the arguments of attn_fwd / attn_bwd_accumulate."""
@@ -310,7 +312,7 @@ def attn_plan(B: int, Hq: int, Hkv: int, D: int, Sq: int, chunk_lens: Sequence[i
     a.B, a.Hq, a.Hkv, a.D, a.Sq, a.n_chunks = B, Hq, Hkv, D, Sq, len(chunk_lens)
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.io_dtype = _DT[dtype]
-    a.flags = _lib.LTR_CAUSAL if causal else 0
+    a.flags = (_lib.LTR_CAUSAL if causal else 0) | (_lib.LTR_FWD_F32_SCALAR if f32_scalar else 0)
     for val, lo, hi, name in ((fwd_rows, _lib.LTR_FWD_ROWS_256, _lib.LTR_FWD_ROWS_512, "fwd_rows"),
                               (dq_rows, _lib.LTR_DQ_ROWS_256, _lib.LTR_DQ_ROWS_512, "dq_rows"),
                               (dkdv_keys, _lib.LTR_DKDV_KEYS_128, _lib.LTR_DKDV_KEYS_256, "dkdv_keys")):

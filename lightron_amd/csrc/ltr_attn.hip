@@ -13,7 +13,9 @@
 //                        with an earlier partial result is part of the epilogue.
 //                        fwd_bf16_kernel<64, 2>: two 32-row blocks per wave (512 rows per block, 64-key tiles): every K / V
 //                        operand read from LDS feeds two MFMAs (chosen by the host, or forced with LTR_FWD_ROWS_512).
-//   fwd_f32_kernel<D>    fp32 I/O and arithmetic (no MFMA), for the 1e-4 parity case.
+//   fwd_f32_mfma_kernel<D, KS>  fp32 I/O and arithmetic on v_mfma_f32_32x32x2_f32: the forward of the 1e-4 cases (the reference's
+//                        acceptance dtype) on the matrix pipe; KS key shares per 32-row group for launches with few rows.
+//   fwd_f32_kernel<D>    the same in scalar fp32 (no MFMA): kept as the fallback, reached with LTR_FWD_F32_SCALAR.
 //   delta_kernel         DELTA = rowsum(dO * O).
 //   bwd_dkdv_kernel<D, KW>  a block of 8 waves owns 128 * KW keys of one kv head and loops over the
 //                        query heads of the GQA group and over 64-row query tiles taken from
@@ -1008,6 +1010,286 @@ __global__ __launch_bounds__(64) void fwd_f32_kernel(const FwdParams p) {
         if (p.flags & LTR_MERGE) val += op[d] * w_old;
         op[d] = val;
     }
+}
+
+// ------------------------------------------------------------------------------ forward, fp32 on the matrix pipe
+// v_mfma_f32_32x32x2_f32 (lane l, i = l % 32, h = l / 32: A[i][h], B[h][i], C as for the bf16 shape): fp32 operands and
+// fp32 accumulation, so the 1e-4 cases run on the matrix pipe at full precision.  A block has 4 waves; a wave owns 32 query
+// rows (a lane = one query, as in the bf16 kernel) and one of KS interleaved shares of the keys: the RG = 4 / KS waves with
+// different rows share every K / V tile, the KS waves with the same rows take the sub-tiles ks, ks + KS, ... of 32 keys and
+// their partial (m, l, O) are merged at the end.  KS > 1 is for launches with too few query rows to fill the device (the
+// reference's acceptance shapes).  Both contractions pick their own order of the contraction index so that no operand moves:
+//   S^T = K Q^T   step 4g + j contracts d = 8g + 4h + j: the K operand of four steps is one 128-bit LDS read, Q stays in
+//                 registers in that order;
+//   O^T += V^T P^T  step r contracts the key of accumulator register r (8 (r / 4) + 4h + r % 4): P^T is used where it is.
+// K / V tiles of 32 * KS keys go global -> LDS directly, double buffered, 16-byte chunks XOR-swizzled (f32_swz) so that the
+// 128-bit K reads (16 rows, same chunk) and the 32-bit V reads (one row per half-wave, rows 4 apart) touch every bank once.
+__device__ __forceinline__ int f32_swz(int row) {   // bits 2 and 3 of the row swapped: rows 4 apart land 32 banks apart
+    return (row & 3) | (((row >> 2) & 1) << 3) | (((row >> 3) & 1) << 2);
+}
+
+template <int D, int KS>
+struct F32Mfma {
+    static constexpr int NW = 4, RG = NW / KS;          // waves; row groups of 32 rows
+    static constexpr int BM = 32 * RG, BN = 32 * KS;    // rows per block, keys per step
+    static constexpr int TILE = BN * D;                 // floats per K (or V) tile
+    static constexpr int BUF_BYTES = 2 * TILE * 4;      // {K tile, V tile}
+    static constexpr int ML_OFF = 0, ML_BYTES = NW * 64 * 4;                        // per wave: m[32], l[32]
+    static constexpr int PART_OFF = ML_BYTES, PART_BYTES = (D / 32) * 16 * 64 * 4;  // one wave's O^T accumulators, lane-major
+    static constexpr int MERGE_BYTES = PART_OFF + (KS - 1) * RG * PART_BYTES;
+    static constexpr int STAGE_OFF = MERGE_BYTES;       // row-major staging of the RG writing waves, after the merge area
+    static constexpr int EPI_BYTES = STAGE_OFF + RG * WaveStage<D>::BYTES;
+    static constexpr int LDS = 2 * BUF_BYTES > EPI_BYTES ? 2 * BUF_BYTES : EPI_BYTES;
+    static_assert(LDS <= 160 * 1024, "LDS of one CU");
+};
+
+template <int D, int KS>
+__global__ __launch_bounds__(256) void fwd_f32_mfma_kernel(const FwdParams p) {
+    using L = F32Mfma<D, KS>;
+    constexpr int NW = L::NW, RG = L::RG, BM = L::BM, BN = L::BN, TILE = L::TILE;
+    constexpr int CPR = D / 4;               // 16-byte chunks per row
+    constexpr int RPI = 64 / CPR;            // rows filled by one wave-wide LDS-direct load (1 KB)
+    constexpr int NI = BN / (RPI * NW);      // such loads per wave, per tensor and per step
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = w / KS, ks = w % KS;
+    const bool causal = p.flags & LTR_CAUSAL;
+    int idx = blockIdx.x;
+    const int qt = p.n_qtiles - 1 - idx / (p.B * p.Hq);     // late (heavier under a causal mask) q tiles first
+    const int bh = idx % (p.B * p.Hq);
+    const int b = bh / p.Hq, h = bh % p.Hq, hkv = h / p.n_rep;
+    const int row0 = qt * BM, my_row = row0 + rg * 32 + l32;
+    const bool row_ok = my_row < p.Sq;
+    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int blk_lo, blk_hi, w_lo, w_hi;
+    q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+    {
+        const int wr0 = row0 + rg * 32, wr1 = min(wr0 + 32, p.Sq) - 1;
+        if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
+        else { w_lo = 0x7fffffff; w_hi = -0x7fffffff; }   // wave has no valid row
+    }
+
+    // Q operand: qreg[4g + j] = Q[row][8g + 4h + j]
+    float qreg[D / 2];
+    {
+        const float *qp = (const float *)p.q + b * p.qs[0] + (long long)min(my_row, p.Sq - 1) * p.qs[1] + h * p.qs[2];
+#pragma unroll
+        for (int g = 0; g < D / 8; g++) {
+            f32x4 x = *(const f32x4 *)(qp + 8 * g + 4 * hh);
+            if (!row_ok) x = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; j++) qreg[4 * g + j] = x[j];
+        }
+    }
+    f32x16 oacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;   // exp2 domain; l_run: this lane's half of the keys
+    const float c2 = p.scale * LTR_LOG2E;
+
+    // step iterator over (chunk, BN keys); chunk fields live in scalar registers (see the bf16 kernel)
+    int c = -1, t = 0, nt = 0;
+    int ld_sk = 0, ld_pos0 = 0;
+    const float *ld_kb = nullptr, *ld_vb = nullptr;
+    auto settle = [&]() {
+        while (c < p.n_chunks && t >= nt) {
+            c++;
+            t = 0;
+            if (c < p.n_chunks) {
+                ld_sk = p.chunk[c].sk;
+                ld_pos0 = p.chunk[c].pos0;
+                ld_kb = (const float *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+                ld_vb = (const float *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+                const int nvis = causal ? max(0, min(ld_sk, blk_hi - ld_pos0 + 1)) : ld_sk;
+                nt = (nvis + BN - 1) / BN;
+            }
+        }
+    };
+    settle();
+    const int st_row = lane / CPR, st_pc = lane % CPR;
+    int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;
+    auto gload = [&](int ti, int buf) {
+        nx_sk = ld_sk;
+        nx_pos0 = ld_pos0;
+        nx_key0 = ti * BN;
+        const unsigned Kd = lds_address(smem) + buf * L::BUF_BYTES, Vd = Kd + TILE * 4;
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const int row = RPI * (NI * w + i) + st_row;
+            const int key = min(ti * BN + row, ld_sk - 1);       // rows past the end repeat the last row; they are masked
+            const int chunk = st_pc ^ f32_swz(row);
+            global_to_lds_b128(ld_kb + ((long long)key * p.ks[1] + chunk * 4), Kd + RPI * (NI * w + i) * D * 4);
+            global_to_lds_b128(ld_vb + ((long long)key * p.vs[1] + chunk * 4), Vd + RPI * (NI * w + i) * D * 4);
+        }
+    };
+    bool have = c < p.n_chunks;
+    if (have) gload(t, 0);
+    tile_barrier();
+    int par = 0;
+    while (have) {
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0 + 32 * ks;   // this wave's 32 keys of the step
+        const float *Ks = (const float *)(smem + par * L::BUF_BYTES) + 32 * ks * D, *Vs = Ks + TILE;
+        t++;
+        settle();
+        const bool have_next = c < p.n_chunks;
+        if (have_next) gload(t, par ^ 1);
+        // nothing to add: the sub-tile starts past the chunk's end, or every row of the wave precedes its first key
+        if (key0 < sk && (!causal || pos0 + key0 <= w_hi)) {
+            f32x16 s;
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[r] = 0.f;
+            const float *krow = Ks + l32 * D;
+            const int ksw = f32_swz(l32);
+#pragma unroll
+            for (int g = 0; g < D / 8; g++) {
+                const f32x4 kx = *(const f32x4 *)(krow + (((2 * g + hh) ^ ksw) << 2));
+#pragma unroll
+                for (int j = 0; j < 4; j++) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[j], qreg[4 * g + j], s, 0, 0, 0);
+            }
+            const bool need_mask = (key0 + 32 > sk) || (causal && (pos0 + key0 + 31 > w_lo));
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float tv = s[r] * c2;
+                if (need_mask) {
+                    const int key = key0 + 8 * (r / 4) + 4 * hh + (r % 4);
+                    const bool vis = key < sk && (!causal || pos0 + key <= my_pos);
+                    tv = vis ? tv : -INFINITY;
+                }
+                s[r] = tv;
+                mx = fmaxf(mx, tv);
+            }
+            mx = xhalf_max(mx);                                   // row max over the 32 keys (both halves agree)
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);   // m_run = -inf: 0 (nothing accumulated yet)
+            float l_tile = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                s[r] = __builtin_amdgcn_exp2f(s[r] - m_use);
+                l_tile += s[r];
+            }
+            l_run = l_run * alpha + l_tile;
+            m_run = m_new;
+#pragma unroll
+            for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+            // O^T += V^T P^T: step r contracts key 8 (r / 4) + 4h + r % 4; lane (d = 32 db + l32, h) reads V[key][d]
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int vrow = 8 * (r / 4) + 4 * hh + (r % 4);
+                const float *vr = Vs + vrow * D + (l32 & 3);
+                const int vsw = f32_swz(vrow);
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    const float vx = vr[((8 * db + (l32 >> 2)) ^ vsw) << 2];
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx, s[r], oacc[db], 0, 0, 0);
+                }
+            }
+        }
+        tile_barrier();
+        par ^= 1;
+        have = have_next;
+    }
+
+    // merge of the KS partial results of a row group (the tile buffers are no longer read: the last barrier is behind us)
+    float l_tot = xhalf_sum(l_run);
+    if constexpr (KS > 1) {
+        float *ml = (float *)(smem + L::ML_OFF);
+        if (hh == 0) {
+            ml[w * 64 + l32] = m_run;
+            ml[w * 64 + 32 + l32] = l_tot;
+        }
+        __syncthreads();
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int k2 = 0; k2 < KS; k2++) m_all = fmaxf(m_all, ml[(rg * KS + k2) * 64 + l32]);
+        const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+        float l_sum = 0.f;
+#pragma unroll
+        for (int k2 = 0; k2 < KS; k2++)
+            l_sum += ml[(rg * KS + k2) * 64 + 32 + l32] * __builtin_amdgcn_exp2f(ml[(rg * KS + k2) * 64 + l32] - m_ref);
+        const float f_own = __builtin_amdgcn_exp2f(m_run - m_ref);
+        float *part = (float *)(smem + L::PART_OFF);
+        if (ks > 0) {
+            float *mine = part + (size_t)(rg * (KS - 1) + ks - 1) * (L::PART_BYTES / 4);
+#pragma unroll
+            for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    f32x4 x;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] = oacc[i][4 * r4 + e] * f_own;
+                    *(f32x4 *)(mine + ((i * 4 + r4) * 64 + lane) * 4) = x;
+                }
+        }
+        __syncthreads();
+        if (ks == 0) {
+#pragma unroll
+            for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][r] *= f_own;
+            for (int k2 = 1; k2 < KS; k2++) {
+                const float *other = part + (size_t)(rg * (KS - 1) + k2 - 1) * (L::PART_BYTES / 4);
+#pragma unroll
+                for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; r4++) {
+                        const f32x4 x = *(const f32x4 *)(other + ((i * 4 + r4) * 64 + lane) * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) oacc[i][4 * r4 + e] += x[e];
+                    }
+            }
+        }
+        m_run = m_all;
+        l_tot = l_sum;
+        if (ks > 0) return;    // no barrier follows
+    }
+
+    // epilogue of the wave that holds the row group's result: normalise, optional merge with (o, lse), whole rows out
+    float lse_new = (l_tot > 0.f) ? m_run * LTR_LN2 + logf(l_tot) : -INFINITY;
+    float w_cur = (l_tot > 0.f) ? 1.f / l_tot : 0.f, w_old = 0.f;
+    float *lse_p = p.lse + ((long long)b * p.Hq + h) * p.Sq + my_row;
+    if ((p.flags & LTR_MERGE) && row_ok) {
+        const float lse_old = *lse_p;
+        const float mxl = fmaxf(lse_old, lse_new);
+        if (mxl == -INFINITY) {
+            w_cur = 0.f;
+        } else {
+            const float e_old = expf(lse_old - mxl), e_new = expf(lse_new - mxl);
+            const float tot = e_old + e_new;
+            w_old = e_old / tot;
+            w_cur *= e_new / tot;
+            lse_new = mxl + logf(tot);
+        }
+    }
+    if (row_ok && hh == 0) *lse_p = lse_new;
+    unsigned char *stage = smem + L::STAGE_OFF + rg * WaveStage<D>::BYTES;
+    float *row_w_old = (float *)(stage + 32 * WaveStage<D>::ROW_BYTES);
+    if (hh == 0) row_w_old[l32] = w_old;
+    constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;
+    const int wave_row0 = row0 + rg * 32;
+    const bool merge = (p.flags & LTR_MERGE) != 0;
+    float *op = (float *)p.o + b * p.os[0] + h * p.os[2] + (long long)(wave_row0 + lane / LPR) * p.os[1] + 4 * (lane % LPR);
+    const long long os1 = p.os[1];
+    const int Sq = p.Sq;
+    wave_tile_rowmajor<D>(stage, lane, oacc, w_cur, [&](int row, int, f32x4 val) {
+        if (wave_row0 + row < Sq) {
+            if (merge) {
+                const f32x4 old = *(const f32x4 *)op;
+                const float wo = row_w_old[row];
+#pragma unroll
+                for (int e = 0; e < 4; e++) val[e] += old[e] * wo;
+            }
+            *(f32x4 *)op = val;
+        }
+        op += ROWS_PER_IT * os1;
+    });
 }
 
 // ------------------------------------------------------------------------------ delta
@@ -2171,7 +2453,17 @@ int enable_large_lds() {
               hipFuncSetAttribute((const void *)bwd_dq_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   dq_lds_bytes<64>()) == hipSuccess &&
               hipFuncSetAttribute((const void *)bwd_dq_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  dq_lds_bytes<64>()) == hipSuccess;
+                                  dq_lds_bytes<64>()) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<128, 1>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<128, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<128, 2>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<64, 1>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<64, 2>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<64, 4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<64, 4>::LDS) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
         return LTR_ELAUNCH;
@@ -2259,16 +2551,29 @@ int q_tile_slots(int n_qtiles, long long blocks_per_tile, bool uneven) {
 // ltr_attn_fwd and for ltr_attn_plan, so the plan a caller is shown is the launch it gets.
 struct FwdPlan {
     bool wide;          // 512-row blocks (two 32-row blocks per wave, head dim 64)
+    int f32_ks;         // fp32: 0 = scalar kernel, else the key shares per row group of fwd_f32_mfma_kernel
     int rows, n_qtiles, n_slots;
     long long blocks;
 };
 FwdPlan plan_fwd(int D, bool f32, unsigned flags, int B, int Hq, int Sq, int q_split, const int *q_pos0, const ChunkDev *chunk,
                  int n_chunks) {
     FwdPlan pl;
+    pl.f32_ks = 0;
     if (f32) {
         pl.wide = false;
-        pl.rows = 64;
-        pl.n_qtiles = pl.n_slots = (Sq + 63) / 64;
+        if (flags & LTR_FWD_F32_SCALAR) {
+            pl.rows = 64;
+        } else {
+            // matrix-pipe kernel: 128 rows per block, or fewer rows and the keys split over 2 / 4 waves of a row group when
+            // the launch has too few rows to give every CU a block (4 key shares need the LDS that only head dim 64 leaves)
+            const int cus = device_cus();
+            const int max_ks = D == 64 ? 4 : 2;
+            int ks = 1;
+            while (ks < max_ks && (long long)((Sq + 128 / ks - 1) / (128 / ks)) * B * Hq < cus) ks *= 2;
+            pl.f32_ks = ks;
+            pl.rows = 128 / ks;
+        }
+        pl.n_qtiles = pl.n_slots = (Sq + pl.rows - 1) / pl.rows;
         pl.blocks = (long long)pl.n_qtiles * B * Hq;
         return pl;
     }
@@ -2417,7 +2722,8 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
     if (!a || !a->q || !a->o || !a->lse) return LTR_EINVAL;
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
-    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q | LTR_FWD_ROWS_256 | LTR_FWD_ROWS_512)) return LTR_EINVAL;
+    if (a->flags & ~(LTR_CAUSAL | LTR_MERGE | LTR_ROPE_Q | LTR_FWD_ROWS_256 | LTR_FWD_ROWS_512 | LTR_FWD_F32_SCALAR)) return LTR_EINVAL;
+    if ((a->flags & LTR_FWD_F32_SCALAR) && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     if ((a->flags & LTR_FWD_ROWS_256) && (a->flags & LTR_FWD_ROWS_512)) return LTR_EINVAL;
     if (a->D != 64 && a->D != 128) return LTR_EUNSUP;
     if (a->io_dtype != LTR_BF16 && a->io_dtype != LTR_F32) return LTR_EUNSUP;
@@ -2494,6 +2800,17 @@ extern "C" int ltr_attn_fwd(const ltr_attn_fwd_args *a, void *stream) {
         if (a->D == 128) return launch((const void *)fwd_bf16_kernel<128, 1>, pl.blocks, 512, fwd_lds_bytes<128>(), st, p);
         if (pl.wide) return launch((const void *)fwd_bf16_kernel<64, 2>, pl.blocks, 512, fwd_lds_bytes<64, 2>(), st, p);
         return launch((const void *)fwd_bf16_kernel<64, 1>, pl.blocks, 512, fwd_lds_bytes<64>(), st, p);
+    }
+    if (pl.f32_ks) {   // fp32 on the matrix pipe; the chunk offsets of its LDS-direct loads are 64-bit, nothing more to check
+        rc = enable_large_lds();
+        if (rc) return rc;
+        if (a->D == 128) {
+            if (pl.f32_ks == 1) return launch((const void *)fwd_f32_mfma_kernel<128, 1>, pl.blocks, 256, F32Mfma<128, 1>::LDS, st, p);
+            return launch((const void *)fwd_f32_mfma_kernel<128, 2>, pl.blocks, 256, F32Mfma<128, 2>::LDS, st, p);
+        }
+        if (pl.f32_ks == 1) return launch((const void *)fwd_f32_mfma_kernel<64, 1>, pl.blocks, 256, F32Mfma<64, 1>::LDS, st, p);
+        if (pl.f32_ks == 2) return launch((const void *)fwd_f32_mfma_kernel<64, 2>, pl.blocks, 256, F32Mfma<64, 2>::LDS, st, p);
+        return launch((const void *)fwd_f32_mfma_kernel<64, 4>, pl.blocks, 256, F32Mfma<64, 4>::LDS, st, p);
     }
     if (a->D == 128) return launch((const void *)fwd_f32_kernel<128>, pl.blocks, 64, 0, st, p);
     return launch((const void *)fwd_f32_kernel<64>, pl.blocks, 64, 0, st, p);
@@ -2712,7 +3029,8 @@ extern "C" int ltr_attn_plan(const ltr_attn_bwd_args *a, ltr_attn_plan_t *out) {
     out->dkdv_keys = b.keys_per_block;
     out->dkdv_blocks = b.kv_blocks;
     if (f32) {
-        snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_f32_kernel<%d>", a->D);
+        if (f.f32_ks) snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_f32_mfma_kernel<%d, %d>", a->D, f.f32_ks);
+        else snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_f32_kernel<%d>", a->D);
         snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_f32_kernel<%d>", a->D);
         snprintf(out->dkdv_kernel, sizeof(out->dkdv_kernel), "bwd_dkdv_f32_kernel<%d, *>", a->D);
     } else {

@@ -14,7 +14,7 @@ import torch
 import torch.nn as nn
 
 from .attention import block_attention
-from .layers import apply_rotary_emb, rope_one, rope_table
+from .layers import rope_one, rope_table
 
 
 class LocalCPGroup:
@@ -131,7 +131,7 @@ class ContextParallelAttention(nn.Module):
             xk = _all_to_all(xk, 2, 1, self.cp_group)
             xv = _all_to_all(xv, 2, 1, self.cp_group)
             qf, kf, vf = (t.reshape(W * B, S_global, -1, D) for t in (xq, xk, xv))
-            qf, kf = apply_rotary_emb(qf, kf, fc) if H == Hkv else _rope_each(qf, kf, fc)
+            qf, kf = rope_one(qf, fc), rope_one(kf, fc)          # one streaming pass per tensor (q and k may differ in heads)
             o, _ = block_attention(qf, [kf], [vf], [0], 0, None, self.causal)
             o = o.view(W, B, S_global, H // W, D)
             o = _all_to_all(o, 1, 2, self.cp_group)              # [W, B, S_local, H, D]
@@ -156,8 +156,3 @@ class ContextParallelAttention(nn.Module):
             o = torch.stack(outs, 0)
         return self.local_attn.wo(o.flatten(3))
 
-
-def _rope_each(q, k, fc):
-    q2, _ = apply_rotary_emb(q, q, fc)
-    k2, _ = apply_rotary_emb(k, k, fc)
-    return q2, k2

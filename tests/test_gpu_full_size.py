@@ -17,12 +17,21 @@ def _rel(a, b):
     return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
 
 
-def _check_rows(q, k, v, qpos, kpos, causal, o, lse, do=None, dq=None, n=24, seed=0):
+def _edges(marks, size, n_b, n_h):
+    """Deterministic samples on both sides of the boundaries in `marks` (tile, half-chunk and segment edges):
+    indices m - 1 and m for every mark inside (0, size), batches and heads taken in turn."""
+    idx = sorted({i for m in marks for i in (m - 1, m) if 0 <= i < size})
+    return [(j % n_b, (3 * j + 1) % n_h, i) for j, i in enumerate(idx)]
+
+
+def _check_rows(q, k, v, qpos, kpos, causal, o, lse, do=None, dq=None, n=24, seed=0, edge_rows=()):
     g = torch.Generator().manual_seed(seed)
     B, Sq, Hq, _ = q.shape
     rows = [(int(torch.randint(B, (1,), generator=g)), int(torch.randint(Hq, (1,), generator=g)),
              int(torch.randint(Sq, (1,), generator=g))) for _ in range(n)]
     rows += [(0, 0, 0), (B - 1, Hq - 1, Sq - 1)]
+    # block edges of the kernels (256-row q tiles: rows 255 / 256) and the caller's own edges (segment split, ragged end)
+    rows += _edges([256, Sq] + list(edge_rows), Sq, B, Hq)
     ref = orc.sampled_rows(q, k, v, qpos, kpos, causal, rows, do)
     num = den = 0.0
     for (b, h, i), (ro, rl, rdq) in zip(rows, ref):
@@ -35,12 +44,15 @@ def _check_rows(q, k, v, qpos, kpos, causal, o, lse, do=None, dq=None, n=24, see
         assert (num / den) ** 0.5 < GRAD_RTOL, ("dQ", (num / den) ** 0.5)
 
 
-def _check_keys(q, k, v, o, lse, do, qpos, kpos, causal, dk, dv, n=6, seed=1):
+def _check_keys(q, k, v, o, lse, do, qpos, kpos, causal, dk, dv, n=6, seed=1, edge_keys=()):
     g = torch.Generator().manual_seed(seed)
     B, Sk, Hkv, _ = k.shape
     keys = [(int(torch.randint(B, (1,), generator=g)), int(torch.randint(Hkv, (1,), generator=g)),
              int(torch.randint(Sk, (1,), generator=g))) for _ in range(n)]
     keys += [(0, 0, 0), (B - 1, Hkv - 1, Sk - 1)]
+    # block edges of the dK/dV kernel (128-key blocks: keys 127 / 128) and the caller's own (chunk and half-chunk boundaries,
+    # the last tile a diagonal sees)
+    keys += _edges([128] + list(edge_keys), Sk, B, Hkv)
     ref = orc.sampled_keys(q, k, v, o, lse, do, qpos, kpos, causal, keys)
     nk = dk_ = nv = dv_ = 0.0
     for (b, gi, j), (rk, rv) in zip(keys, ref):
@@ -120,8 +132,11 @@ def test_config3_full_all_ranks(ltr, path):
         dk[:, rp[r].cuda()], dv[:, rp[r].cuda()] = dk_acc[r], dv_acc[r]
     pos = torch.arange(S)
     oc, lsec, dqc, dkc, dvc = o.cpu(), lse.cpu(), dq.cpu(), dk.cpu(), dv.cpu()
-    _check_rows(q, k, v, pos, pos, True, oc, lsec, do, dqc, n=30)
-    _check_keys(q, k, v, oc, lsec, do, pos, pos, True, dkc, dvc, n=6)
+    # edges: every half-chunk boundary (first / last key of each half-chunk; for rows, the segment split of the rank that
+    # owns them), and a key inside the last 64-key tile that the diagonal of the last half-chunk sees
+    half = [i * hc for i in range(1, 2 * W)]
+    _check_rows(q, k, v, pos, pos, True, oc, lsec, do, dqc, n=30, edge_rows=[hc, S // 2, S - hc])
+    _check_keys(q, k, v, oc, lsec, do, pos, pos, True, dkc, dvc, n=6, edge_keys=half + [S - 63])
     # softmax rows sum to one: sum_j dV_j == sum over the group's query heads and rows of dO
     lhs = dvc.double().sum(1)                                            # [B,Hkv,D]
     rhs = do.double().sum(1).reshape(B, Hkv, Hq // Hkv, D).sum(2)
@@ -155,8 +170,9 @@ def test_config3_full_ring_entry_point_fp32_kv_grads(ltr):
     for r in range(W):
         dk[:, rp[r]], dv[:, rp[r]] = kv[r][0].grad.cpu(), kv[r][1].grad.cpu()
     pos = torch.arange(S)
-    _check_rows(q, k, v, pos, pos, True, o, lse, do, dq, n=20, seed=3)
-    _check_keys(q, k, v, o, lse, do, pos, pos, True, dk, dv, n=6, seed=4)
+    hc = S // (2 * W)
+    _check_rows(q, k, v, pos, pos, True, o, lse, do, dq, n=20, seed=3, edge_rows=[hc, S // 2, S - hc])
+    _check_keys(q, k, v, o, lse, do, pos, pos, True, dk, dv, n=6, seed=4, edge_keys=[i * hc for i in range(1, 2 * W, 3)] + [S - 63])
     rhs = do.double().sum(1).reshape(B, Hkv, Hq // Hkv, D).sum(2)
     assert _rel(dv.double().sum(1), rhs) < 1e-2
 
@@ -226,8 +242,10 @@ def test_config4_full_rank15(ltr, path):
     qpos, kpos = torch.arange(sl) + 15 * sl, torch.arange(S)
     qc = q[:, 15 * sl:]
     oc, lsec = ol.cpu(), lsel.cpu()
-    _check_rows(qc, k, v, qpos, kpos, True, oc, lsec, do, dq.cpu(), n=20)
-    _check_keys(qc, k, v, oc, lsec, do, qpos, kpos, True, dk.cpu(), dv.cpu(), n=6)
+    # edges: chunk boundaries of the ring (first / last key of a chunk), the first key of the diagonal chunk and a key in
+    # the last tile the diagonal sees
+    _check_rows(qc, k, v, qpos, kpos, True, oc, lsec, do, dq.cpu(), n=20, edge_rows=[sl // 2])
+    _check_keys(qc, k, v, oc, lsec, do, qpos, kpos, True, dk.cpu(), dv.cpu(), n=6, edge_keys=[sl, 8 * sl, 15 * sl, S - 63])
 
 
 def test_config5_full_ulysses_layout(ltr):
@@ -296,8 +314,9 @@ def test_head_dim_64_ring_share_both_block_sizes(ltr, keys, rows):
     ltr.attn_bwd_accumulate(ql, dol, lsel, delta_ws, ks, vs, pos0, dq, dks, dvs, qp, hc, True, do_dq=False, dkdv_keys=keys)
     kpos = torch.arange(S)
     oc, lsec = ol.cpu(), lsel.cpu()
-    _check_rows(q[:, qpos], k, v, qpos, kpos, True, oc, lsec, do, dq.cpu(), n=20)
-    _check_keys(q[:, qpos], k, v, oc, lsec, do, qpos, kpos, True, dk.cpu(), dv.cpu(), n=8)
+    # edges: the segment split of the share's rows (q_split - 1 / q_split), 512-row tile edges, half-chunk boundaries of the keys
+    _check_rows(q[:, qpos], k, v, qpos, kpos, True, oc, lsec, do, dq.cpu(), n=20, edge_rows=[hc, 512])
+    _check_keys(q[:, qpos], k, v, oc, lsec, do, qpos, kpos, True, dk.cpu(), dv.cpu(), n=8, edge_keys=[256, 3 * hc, 6 * hc, 6 * hc - 63])
 
 
 @pytest.mark.parametrize("Sq", [2048, 1900])
@@ -324,5 +343,5 @@ def test_head_dim_64_paired_512_row_blocks(ltr, Sq):
     ltr.attn_bwd_accumulate(qd, dod, lse, delta_ws, [kd], [vd], [0], dq, [dk], [dv], 0, None, True, do_dq=False)
     pos = torch.arange(Sq)
     oc, lsec = o.cpu(), lse.cpu()
-    _check_rows(q, k, v, pos, pos, True, oc, lsec, do, dq.cpu(), n=30)
-    _check_keys(q, k, v, oc, lsec, do, pos, pos, True, dk.float().cpu(), dv.float().cpu(), n=8)
+    _check_rows(q, k, v, pos, pos, True, oc, lsec, do, dq.cpu(), n=30, edge_rows=[512, Sq - Sq % 512 or Sq])
+    _check_keys(q, k, v, oc, lsec, do, pos, pos, True, dk.float().cpu(), dv.float().cpu(), n=8, edge_keys=[256, Sq - 63])

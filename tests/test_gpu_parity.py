@@ -94,6 +94,48 @@ def test_reference_acceptance_noncausal_fp32(ltr):
     assert (torch.cat(outs, 1).cpu() - ref).abs().max() < F32_TOL
 
 
+@pytest.mark.parametrize("D,B,Hq,Hkv,Sq,q_pos,split,chunks,causal,want", [
+    (64, 2, 8, 8, 256, (768, 768), None, [(768, 256), (512, 256), (256, 256), (0, 256)], True, "fwd_f32_mfma_kernel<64, 4>"),   # config 1, rank 3
+    (64, 2, 8, 8, 8, (0, 0), None, [(0, 8), (24, 8), (16, 8), (8, 8)], False, "fwd_f32_mfma_kernel<64, 4>"),   # the reference's acceptance shape
+    (64, 4, 16, 4, 300, (100, 900), 130, [(0, 200), (200, 333), (533, 700)], True, "fwd_f32_mfma_kernel<64, 2>"),   # ragged, GQA, two-segment rows
+    (64, 2, 16, 16, 1024, (0, 0), None, [(0, 1024)], True, "fwd_f32_mfma_kernel<64, 1>"),
+    (128, 1, 4, 2, 200, (56, 56), None, [(0, 100), (100, 156)], True, "fwd_f32_mfma_kernel<128, 2>"),
+    (128, 4, 16, 4, 520, (0, 0), None, [(0, 260), (260, 300)], False, "fwd_f32_mfma_kernel<128, 1>"),
+])
+def test_fp32_forward_on_the_matrix_pipe(ltr, D, B, Hq, Hkv, Sq, q_pos, split, chunks, causal, want):
+    """The fp32 forward on v_mfma_f32_32x32x2_f32 in every instantiation (1, 2 or 4 key shares per row group, chosen by
+    the library from the launch's rows: the plan must name the expected kernel on a 256-CU device), against the dense
+    oracle to 1e-4 on O and LSE, in one launch and step by step with the merge epilogue, and against the scalar fp32
+    kernel (LTR_FWD_F32_SCALAR)."""
+    plan = ltr.attn_plan(B, Hq, Hkv, D, Sq, [n for _, n in chunks], [p0 for p0, _ in chunks], q_pos, split, causal, dtype=torch.float32)
+    if plan["compute_units"] == 256:
+        assert plan["fwd"]["kernel"] == want
+    assert plan["fwd"]["kernel"].startswith("fwd_f32_mfma_kernel")
+    assert ltr.attn_plan(B, Hq, Hkv, D, Sq, [n for _, n in chunks], [p0 for p0, _ in chunks], q_pos, split, causal,
+                         dtype=torch.float32, f32_scalar=True)["fwd"]["kernel"] == "fwd_f32_kernel<%d>" % D
+    g = torch.Generator().manual_seed(4000 + Sq + D)
+    sp = Sq if split is None else split
+    qpos = torch.cat([torch.arange(sp) + q_pos[0], torch.arange(Sq - sp) + q_pos[1]])
+    q = _randn((B, Sq, Hq, D), g, torch.float32)
+    ks = [_randn((B, n, Hkv, D), g, torch.float32) for _, n in chunks]
+    vs = [_randn((B, n, Hkv, D), g, torch.float32) for _, n in chunks]
+    kpos = torch.cat([torch.arange(n) + p0 for p0, n in chunks])
+    o_ref, lse_ref = orc.dense_attention(q, torch.cat(ks, 1), torch.cat(vs, 1), qpos, kpos, causal)
+    qd, kd, vd = q.cuda(), [k.cuda() for k in ks], [v.cuda() for v in vs]
+    pos0 = [p0 for p0, _ in chunks]
+    o, lse = ltr.attn_fwd(qd, kd, vd, pos0, q_pos, split, causal)
+    o_sc, lse_sc = ltr.attn_fwd(qd, kd, vd, pos0, q_pos, split, causal, f32_scalar=True)
+    o_st, lse_st = ltr.attn_fwd(qd, kd[:1], vd[:1], pos0[:1], q_pos, split, causal)
+    for i in range(1, len(chunks)):
+        ltr.attn_fwd(qd, kd[i:i + 1], vd[i:i + 1], pos0[i:i + 1], q_pos, split, causal, out=o_st, lse=lse_st, merge=True)
+    fin = torch.isfinite(lse_ref)
+    for oo, ll in ((o, lse), (o_sc, lse_sc), (o_st, lse_st)):
+        assert (oo.cpu().double() - o_ref).abs().max() < F32_TOL
+        assert torch.equal(torch.isfinite(ll.cpu()), fin)
+        assert (ll.cpu().double()[fin] - lse_ref[fin]).abs().max() < F32_TOL
+    assert (o - o_sc).abs().max() < 2e-5
+
+
 def test_config2_shape_scaled_multi_chunk_bf16(ltr):
     """Config 2 at reduced B/H: last rank's Q chunk of 1024 against 8 KV chunks of 1024, bf16, causal,
     inputs N(0,1)*0.5, fused and step-wise (merge epilogue) paths."""
@@ -837,10 +879,12 @@ def test_paired_q_tiles_forward_backward(ltr, D, B, Hq, Hkv, Sq, q_pos, split, c
     per block (q_tile_slots: causal, and the equal blocks fill the 256 CUs evenly).  Odd tile counts (the middle tile runs
     alone), a ragged last tile, GQA, both head dims, two-segment rows; against the dense oracle."""
     g = torch.Generator().manual_seed(77 + Sq)
+    # the library itself says whether it pairs the tiles of this launch (for the device this test runs on)
+    plan = ltr.attn_plan(B, Hq, Hkv, D, Sq, [n for _, n in chunks], [p0 for p0, _ in chunks], q_pos, split, True)
     n_qt = (Sq + 255) // 256
-    n_slots = (n_qt + 1) // 2
-    blocks = n_slots * B * Hq
-    assert blocks * 10 >= -(-blocks // 256) * 256 * 9, "shape does not trigger the pairing"
+    assert plan["fwd"]["rows"] == plan["dq"]["rows"] == 256
+    assert plan["fwd"]["paired"] and plan["dq"]["paired"], "shape does not trigger the pairing on this device"
+    assert plan["fwd"]["blocks"] == plan["dq"]["blocks"] == ((n_qt + 1) // 2) * B * Hq
     sp = Sq if split is None else split
     qpos = torch.cat([torch.arange(sp) + q_pos[0], torch.arange(Sq - sp) + q_pos[1]])
     q, do = _randn((B, Sq, Hq, D), g, torch.bfloat16), _randn((B, Sq, Hq, D), g, torch.bfloat16)
