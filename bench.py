@@ -673,7 +673,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "s2k", "rope", "mfma_ceiling", "c3_stepwise", "c1", "ref_default"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other workloads and the device probe")
     args = ap.parse_args()
@@ -689,6 +689,12 @@ def main():
         return _bench_mfma_ceiling(args)
     la._lib.load()
     torch.cuda.set_device(0)
+    if args.workload in ("c3_stepwise", "c1", "ref_default"):
+        # side workloads on their own (for profiles): the entry that the default run reports under other_workloads
+        fn = {"c3_stepwise": lambda: _run_c3_stepwise(la, torch, args.steps, args.warmup), "c1": lambda: _run_c1(la, torch),
+              "ref_default": lambda: _run_ref_default(la, torch)}[args.workload]
+        print(json.dumps({"workload": args.workload, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "result": fn()}), flush=True)
+        return
     cfg = _workload(args.workload)
     # the headline workload: exactly --warmup untimed and --steps timed steps (35 ms each: the device has settled after
     # the warm-up); the sub-millisecond workloads warm up for at least 0.3 s ("warmup" reports the steps that took)

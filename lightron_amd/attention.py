@@ -542,6 +542,44 @@ class SingleChunkAttentionFunction(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+_warned_pad = False
+
+
+def _padded_head_dim(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, kv_grad_acc, q_rope):
+    """Head dims the kernels are not instantiated for (anything but 64 and 128; the reference hands any dim // n_heads to
+    SDPA, model/model.py:135, 193): a SLOW PATH that zero-pads q, k and v to the next instantiated head dim (one copy of
+    each tensor per call, the gradients sliced back by autograd), keeps the scale of the TRUE head dim, and slices the
+    result.  Zero columns change neither the scores nor the real columns of O.  Multiples of 8 up to 128."""
+    D = q.shape[-1]
+    if D > 128 or D % 8 or D <= 0:
+        raise RuntimeError("head dim %d: the HIP kernels exist for 64 and 128; other head dims are zero-padded up to the "
+                           "next of the two, which needs a multiple of 8 that is at most 128" % D)
+    if kv_grad_acc is not None:
+        raise RuntimeError("kv_grad_acc accumulators are shaped like the un-padded chunks: not available with a padded head dim")
+    global _warned_pad
+    if not _warned_pad:
+        _warned_pad = True
+        import warnings
+        warnings.warn("lightron_amd: head dim %d is zero-padded to %d on every call (a copy of q, k and v)"
+                      % (D, 64 if D < 64 else 128), stacklevel=3)
+    Dp = 64 if D < 64 else 128
+    pad = (0, Dp - D)
+    lens = [k.shape[1] for k in ks]
+    kbuf = torch.nn.functional.pad(ks[0] if len(ks) == 1 else torch.cat(list(ks), 1), pad)
+    vbuf = torch.nn.functional.pad(vs[0] if len(vs) == 1 else torch.cat(list(vs), 1), pad)
+    offs = [sum(lens[:i]) for i in range(len(lens))]
+    ksp = [kbuf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+    vsp = [vbuf[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+    if q_rope is not None:
+        # the padded pairs are rotated by the identity (cos, sin) = (1, 0)
+        ident = torch.zeros((q_rope.shape[0], (Dp - D) // 2, 2), dtype=q_rope.dtype, device=q_rope.device)
+        ident[..., 0] = 1.0
+        q_rope = torch.cat([q_rope, ident], 1).contiguous()
+    o, lse = block_attention(torch.nn.functional.pad(q, pad), ksp, vsp, k_pos0, q_pos0, q_split, causal,
+                             scale if scale is not None else 1.0 / math.sqrt(D), stepwise, out_dtype, None, q_rope)
+    return o[..., :D], lse
+
+
 def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, scale=None, stepwise=False,
                     out_dtype=None, kv_grad_acc=None, q_rope=None):
     """Differentiable entry: returns (O, LSE).  q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table indexed by global
@@ -552,6 +590,8 @@ def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, sca
     accumulators makes the one final cast.  That is how a ring sums dK / dV over its ranks without a bf16 rounding
     per rank."""
     n = len(ks)
+    if q.shape[-1] not in (64, 128):
+        return _padded_head_dim(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, stepwise, out_dtype, kv_grad_acc, q_rope)
     if (n == 1 and kv_grad_acc is None and not stepwise and q.dtype == torch.bfloat16 and out_dtype in (None, torch.bfloat16)
             and q.is_cuda and ks[0].is_cuda and vs[0].is_cuda):
         if isinstance(q_pos0, (tuple, list)):

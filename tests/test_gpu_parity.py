@@ -407,6 +407,43 @@ def test_rope_kernel_bit_exact(ltr, dtype):
         ltr.apply_rotary_emb(x.cuda().transpose(1, 2), x.cuda().transpose(1, 2), fc.cuda()[:8])
 
 
+@pytest.mark.parametrize("D,Hq,Hkv,dtype,causal", [(96, 4, 2, torch.bfloat16, True), (32, 2, 2, torch.bfloat16, False),
+                                                     (80, 4, 4, torch.bfloat16, True), (40, 2, 1, torch.float32, True)])
+def test_other_head_dims_take_the_padded_path(ltr, D, Hq, Hkv, dtype, causal):
+    """Head dims other than 64 / 128 (the reference takes any dim // n_heads, model/model.py:135): block_attention
+    zero-pads them to the next instantiated head dim and keeps the scale 1/sqrt(D) of the true one.  Two ragged chunks,
+    GQA, forward and all three gradients against the dense oracle; head dims the padded path cannot serve are refused."""
+    g = torch.Generator().manual_seed(300 + D)
+    B, Sq, lens, starts = 2, 150, [70, 130], [0, 70]
+    qp = 50
+    q, do = _randn((B, Sq, Hq, D), g, dtype), _randn((B, Sq, Hq, D), g, dtype)
+    ks = [_randn((B, n, Hkv, D), g, dtype) for n in lens]
+    vs = [_randn((B, n, Hkv, D), g, dtype) for n in lens]
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = orc.dense_attention_grads(
+        q.float(), torch.cat(ks, 1).float(), torch.cat(vs, 1).float(), do.float(), torch.arange(Sq) + qp, torch.arange(200), causal,
+        dtype=torch.float32)
+    qd = q.cuda().requires_grad_(True)
+    kd = [k.cuda().requires_grad_(True) for k in ks]
+    vd = [v.cuda().requires_grad_(True) for v in vs]
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")          # the slow path announces itself once per process
+        o, lse = ltr.block_attention(qd, kd, vd, starts, qp, None, causal)
+    o.backward(do.cuda())
+    assert o.shape == (B, Sq, Hq, D)
+    f32 = dtype == torch.float32
+    assert (o.detach().cpu().float() - o_ref).abs().max() < (F32_TOL if f32 else O_TOL_BF16)
+    assert (lse.cpu() - lse_ref).abs().max() < (F32_TOL if f32 else LSE_TOL_BF16)
+    tol = 1e-3 if f32 else GRAD_RTOL_BF16
+    assert _rel(qd.grad.cpu(), dq_ref) < tol
+    assert _rel(torch.cat([k.grad for k in kd], 1).cpu(), dk_ref) < tol
+    assert _rel(torch.cat([v.grad for v in vd], 1).cpu(), dv_ref) < tol
+    for bad in (136, 100):
+        x = torch.zeros(1, 8, 2, bad, dtype=torch.bfloat16, device="cuda")
+        with pytest.raises(RuntimeError, match="head dim"):
+            ltr.block_attention(x, [x], [x], [0])
+
+
 @pytest.mark.gpu
 def test_attention_layer_gqa(ltr):
     """lightron_amd.Attention (model/model.py:123-202 on the HIP kernels) against the reference composition restated
