@@ -670,6 +670,9 @@ __global__ __launch_bounds__(512) void fwd_bf16_kernel(const FwdParams p) {
     // Double-buffered LDS, one barrier per tile: tile t+1 streams into the other buffer (whose readers all
     // passed the previous barrier) while tile t is computed; the barrier also waits for those loads.
     bool have = c < p.n_chunks;
+    // Merging an empty partial result leaves (O, LSE) as they are: a block that sees no key of this launch's chunks (the
+    // early rows of a causal ring step) skips the read-modify-write of its rows altogether.
+    if (!have && (p.flags & LTR_MERGE)) continue;
     if (have) {
         gload_begin(t);
 #pragma unroll
@@ -1127,6 +1130,7 @@ __global__ __launch_bounds__(256) void fwd_f32_mfma_kernel(const FwdParams p) {
         }
     };
     bool have = c < p.n_chunks;
+    if (!have && (p.flags & LTR_MERGE)) return;   // merging an empty partial result changes nothing (block-uniform)
     if (have) gload(t, 0);
     tile_barrier();
     int par = 0;
@@ -2001,6 +2005,15 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     for (int rb = 0; rb < RB; rb++)
 #pragma unroll
         for (int i = 0; i < D / 32; i++) dqacc[rb][i] = zero16;
+    // the dP^T accumulators start at -DELTA of the lane's row (the first MFMA of the chain takes this as its addend), so
+    // dS = P * (dP - DELTA) needs no subtraction per element (one row block per wave only: with two the 16 registers per
+    // row block are not there)
+    constexpr bool DLT_INIT = RB == 1;
+    f32x16 ndlt[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) ndlt[rb][r] = DLT_INIT ? -dlt[rb] : 0.f;
     const float c2 = p.scale * LTR_LOG2E;
 
     // The fields of the chunk being loaded live in scalar registers and are re-read from the argument
@@ -2044,6 +2057,8 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
     };
 
     bool have = c < p.n_chunks;
+    // a block that sees no key of this launch's chunks adds nothing to an fp32 dQ accumulator: no read-modify-write
+    if (!have && !(p.flags & LTR_DQ_BF16)) continue;
     if (have) gload(t, 0);
     tile_barrier();
     // LDS byte addresses of this lane's operands in the K tile of the current buffer (the V tile and the other 32-key
@@ -2083,7 +2098,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
             for (int rb = 0; rb < RB; rb++) {
                 s[rb] = zero16;
-                dp[rb] = zero16;
+                dp[rb] = ndlt[rb];
             }
             __builtin_amdgcn_s_setprio(1);   // MFMA sections run at raised priority, see the forward kernel
             lds_gemm_pair_at_rb<D, RB>(pa, nb * 32 * D * 2, TILE * 2 + nb * 32 * D * 2, qreg, doreg, s, dp);
@@ -2111,7 +2126,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(const BwdParams p) {
                     for (int e = 0; e < 2; e++) {
                         const int r = 2 * j + e;
                         const float pv = __builtin_amdgcn_exp2f(s[rb][r] * c2 - lse2[rb]);
-                        dsv[e] = pv * (dp[rb][r] - dlt[rb]);
+                        dsv[e] = DLT_INIT ? pv * dp[rb][r] : pv * (dp[rb][r] - dlt[rb]);
                     }
                     ds.u[j] = pack2_bf16(dsv[0], dsv[1]);
                 }
