@@ -529,16 +529,17 @@ def _run_c3_stepwise(la, torch, steps, warmup):
     delta = torch.empty(B, Hq, sl, dtype=torch.float32, device=dev)
     n = len(ks)
 
-    def stepwise_fwd():
-        la.attn_fwd(q, ks[:1], vs[:1], pos[:1], qp, qsplit, True, out=o32, lse=lse)
-        for i in range(1, n):
-            la.attn_fwd(q, ks[i:i + 1], vs[i:i + 1], pos[i:i + 1], qp, qsplit, True, out=o32, lse=lse, merge=True)
+    def stepwise_fwd(g_=1):
+        # g_ KV half-chunks per launch: 1 = one launch per half-chunk (16 steps), 2 = one per rank chunk (the 8 steps of this ring)
+        la.attn_fwd(q, ks[:g_], vs[:g_], pos[:g_], qp, qsplit, True, out=o32, lse=lse)
+        for i in range(g_, n, g_):
+            la.attn_fwd(q, ks[i:i + g_], vs[i:i + g_], pos[i:i + g_], qp, qsplit, True, out=o32, lse=lse, merge=True)
 
-    def stepwise_bwd():
+    def stepwise_bwd(g_=1):
         dq32.zero_(); dk32.zero_(); dv32.zero_()
         d = la.attn_delta(o32, do)
-        for i in range(n):
-            la.attn_bwd_accumulate(q, do, lse, d, ks[i:i + 1], vs[i:i + 1], pos[i:i + 1], dq32, dks[i:i + 1], dvs[i:i + 1], qp, qsplit, True)
+        for i in range(0, n, g_):
+            la.attn_bwd_accumulate(q, do, lse, d, ks[i:i + g_], vs[i:i + g_], pos[i:i + g_], dq32, dks[i:i + g_], dvs[i:i + g_], qp, qsplit, True)
         la.cast_to_bf16(dq32); la.cast_to_bf16(dk32); la.cast_to_bf16(dv32)
 
     def table_fwd():
@@ -565,7 +566,8 @@ def _run_c3_stepwise(la, torch, steps, warmup):
     res = {}
     for _ in range(2):
         for key, fn in (("table_fwd_ms", table_fwd), ("table_bwd_ms", table_bwd), ("stepwise_fwd_ms", stepwise_fwd),
-                        ("stepwise_bwd_ms", stepwise_bwd)):
+                        ("stepwise_bwd_ms", stepwise_bwd), ("rank_chunk_steps_fwd_ms", lambda: stepwise_fwd(2)),
+                        ("rank_chunk_steps_bwd_ms", lambda: stepwise_bwd(2))):
             ms = timed(fn)
             res[key] = min(ms, res.get(key, ms))
     pairs = _n_pairs(cfg, r)
@@ -574,10 +576,14 @@ def _run_c3_stepwise(la, torch, steps, warmup):
     out = {"what": "config 3, rank 0's share: one launch per ring step (16 forward launches with LTR_MERGE into fp32 O/LSE, 16 "
                    "ltr_attn_bwd calls into fp32 dQ/dK/dV, zero-fills, DELTA pass and casts included) beside one launch per "
                    "kernel over the 16-entry chunk table",
-           "launches_per_share": {"stepwise": 16 + 1 + 2 * 16 + 6, "table": 1 + 2 + 4}}
+           "launches_per_share": {"stepwise": 16 + 1 + 2 * 16 + 6, "rank_chunk_steps": 8 + 1 + 2 * 8 + 6, "table": 1 + 2 + 4}}
     out.update({key: round(val, 4) for key, val in res.items()})
+    t_rank = res["rank_chunk_steps_fwd_ms"] + res["rank_chunk_steps_bwd_ms"]
     out.update({"stepwise_ms": round(t_step, 4), "table_ms": round(t_tab, 4), "stepwise_over_table": round(t_step / t_tab, 4),
-                "stepwise_tflops": round(f_share / t_step / 1e9, 1), "table_tflops": round(f_share / t_tab / 1e9, 1)})
+                "stepwise_tflops": round(f_share / t_step / 1e9, 1), "table_tflops": round(f_share / t_tab / 1e9, 1),
+                # the same with one launch per RANK chunk (both half-chunks of a rank in one chunk table): the 8 steps of this ring
+                "rank_chunk_steps_ms": round(t_rank, 4), "rank_chunk_steps_over_table": round(t_rank / t_tab, 4),
+                "rank_chunk_steps_tflops": round(f_share / t_rank / 1e9, 1)})
     return out
 
 
