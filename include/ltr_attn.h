@@ -67,6 +67,8 @@ extern "C" {
 
 #define LTR_FWD_F32_SCALAR 32768u /* forward, fp32 only: run the scalar fp32 kernel instead of the matrix-pipe one (same results to
                                     rounding; the fallback and cross-check of fwd_f32_mfma_kernel) */
+#define LTR_BWD_F32_SCALAR 65536u /* backward, fp32 only: the scalar fp32 kernels instead of the matrix-pipe ones (fallback and
+                                    cross-check) */
 
 /* error codes */
 #define LTR_OK 0
@@ -196,8 +198,8 @@ typedef struct ltr_attn_bwd_args {
     int64_t q_split;
     float scale;
     uint32_t flags;       /* LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ |
-                             LTR_DKDV_KEYS_128 | LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_256 | LTR_DQ_ROWS_512 */
-    int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: scalar fp32 kernels for the 1e-4 parity cases;
+                             LTR_DKDV_KEYS_128 | LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_256 | LTR_DQ_ROWS_512 | LTR_BWD_F32_SCALAR */
+    int32_t io_dtype;     /* LTR_BF16 or LTR_F32, of q/k/v/dO (LTR_F32: fp32 kernels on v_mfma_f32_32x32x2_f32 for the 1e-4 cases;
                              LTR_DQ_BF16, LTR_DELTA_FROM_O and LTR_DKDV_BF16 are bf16 only and return LTR_EUNSUP with it) */
     int32_t n_chunks;
     ltr_kv_chunk chunk[LTR_MAX_CHUNKS];

@@ -18,6 +18,7 @@ LTR_DKDV_KEYS_128, LTR_DKDV_KEYS_256 = 512, 1024
 LTR_DQ_ROWS_256, LTR_DQ_ROWS_512 = 2048, 4096
 LTR_FWD_ROWS_256, LTR_FWD_ROWS_512 = 8192, 16384
 LTR_FWD_F32_SCALAR = 32768
+LTR_BWD_F32_SCALAR = 65536
 
 EXPORTS = ("ltr_attn_fwd", "ltr_attn_bwd_delta", "ltr_attn_bwd", "ltr_attn_bwd_noalloc", "ltr_attn_plan", "ltr_cast_f32_to_bf16",
            "ltr_rope_apply", "ltr_abi_version", "ltr_strerror")

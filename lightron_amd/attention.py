@@ -202,7 +202,7 @@ def attn_delta(o: torch.Tensor, do: torch.Tensor) -> torch.Tensor:
 
 def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_accs, q_pos0=0, q_split=None,
                         causal=False, scale=None, do_dq=True, do_dkdv=True, o=None, library_scratch=False, dq_rope=None,
-                        dkdv_keys=None, dq_rows=None):
+                        dkdv_keys=None, dq_rows=None, f32_scalar=False):
     """Adds this Q chunk's contribution into the fp32 accumulators dq_acc / dk_accs / dv_accs.
     do_dq / do_dkdv select which of the two backward kernels are enqueued.  dq_acc may instead be a bf16
     tensor: it then RECEIVES dQ (LTR_DQ_BF16), which is only right when ks / vs hold every KV chunk these
@@ -217,7 +217,8 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     dq_rope: the (cos, sin) table of attn_fwd's q_rope; q is then the ROTATED q (q_rot_out of that forward) and the dQ
     kernel's epilogue rotates dQ back by the conjugate angles (LTR_ROPE_DQ): dq is the gradient of the un-rotated q.
     dkdv_keys: None (the library chooses), 128 or 256 keys per block of the dK/dV kernel (256: bf16 with head dim 64 only).
-    dq_rows: None, 256 or 512 query rows per block of the dQ kernel (512: bf16 with head dim 64 only)."""
+    dq_rows: None, 256 or 512 query rows per block of the dQ kernel (512: bf16 with head dim 64 only).
+    f32_scalar: fp32 inputs only - the scalar fp32 kernels instead of the matrix-pipe ones (LTR_BWD_F32_SCALAR)."""
     lib = _lib.load()
     if library_scratch and (o is None or not do_dq):
         raise RuntimeError("library_scratch needs o (DELTA is computed from it) and do_dq")
@@ -259,7 +260,7 @@ def attn_bwd_accumulate(q, do, lse, delta, ks, vs, k_pos0, dq_acc, dk_accs, dv_a
     a.scale = float(scale if scale is not None else 1.0 / math.sqrt(D))
     a.flags = ((_lib.LTR_CAUSAL if causal else 0) | (0 if do_dq else _lib.LTR_NO_DQ)
                | (0 if do_dkdv else _lib.LTR_NO_DKDV) | (_lib.LTR_DQ_BF16 if dq_direct else 0)
-               | (_lib.LTR_DKDV_BF16 if dkdv_direct else 0))
+               | (_lib.LTR_DKDV_BF16 if dkdv_direct else 0) | (_lib.LTR_BWD_F32_SCALAR if f32_scalar else 0))
     a.io_dtype = _DT[q.dtype]
     if dkdv_keys is not None:
         if dkdv_keys not in (128, 256):
@@ -312,7 +313,7 @@ def attn_plan(B: int, Hq: int, Hkv: int, D: int, Sq: int, chunk_lens: Sequence[i
     a.B, a.Hq, a.Hkv, a.D, a.Sq, a.n_chunks = B, Hq, Hkv, D, Sq, len(chunk_lens)
     a.q_pos0, a.q_split = _qpos(q_pos0, Sq, q_split)
     a.io_dtype = _DT[dtype]
-    a.flags = (_lib.LTR_CAUSAL if causal else 0) | (_lib.LTR_FWD_F32_SCALAR if f32_scalar else 0)
+    a.flags = (_lib.LTR_CAUSAL if causal else 0) | ((_lib.LTR_FWD_F32_SCALAR | _lib.LTR_BWD_F32_SCALAR) if f32_scalar else 0)
     for val, lo, hi, name in ((fwd_rows, _lib.LTR_FWD_ROWS_256, _lib.LTR_FWD_ROWS_512, "fwd_rows"),
                               (dq_rows, _lib.LTR_DQ_ROWS_256, _lib.LTR_DQ_ROWS_512, "dq_rows"),
                               (dkdv_keys, _lib.LTR_DKDV_KEYS_128, _lib.LTR_DKDV_KEYS_256, "dkdv_keys")):

@@ -35,8 +35,10 @@
 //                        bitwise reproducible.  bwd_dq_kernel<64, 2>: two 32-row blocks per wave (a lane owns two
 //                        query rows): every K / V operand read from LDS feeds two MFMAs; head dim 64 only, chosen by the
 //                        host when the wider blocks still fill the device (or forced with LTR_DQ_ROWS_512).
+//   bwd_dq_f32_mfma_kernel<D, KS>, bwd_dkdv_f32_mfma_kernel<D>
+//                        the fp32 backward on v_mfma_f32_32x32x2_f32 (see there).
 //   bwd_dq_f32_kernel<D>, bwd_dkdv_f32_kernel<D, DV>
-//                        the same backward in scalar fp32 (no MFMA), for the 1e-4 parity cases.
+//                        the same backward in scalar fp32 (no MFMA): the fallback, reached with LTR_BWD_F32_SCALAR.
 //   The tile loops of the bf16 kernels are unrolled over their LDS buffers (or, where registers are short,
 //   keep per-lane LDS addresses in registers): no address arithmetic is left between the MFMAs.
 //   RoPE: with LTR_ROPE_Q the forward rotates each q row in its operand registers (rope_rotate8) and can store the
@@ -2405,6 +2407,404 @@ __global__ __launch_bounds__(64) void bwd_dkdv_f32_kernel(const BwdParams p) {
     }
 }
 
+// ------------------------------------------------------------------------------ backward, fp32 on the matrix pipe
+// The recompute backward of the fp32 path on v_mfma_f32_32x32x2_f32, in the shapes of fwd_f32_mfma_kernel (same LDS-direct
+// swizzled fp32 tiles, same choice of contraction order so that no operand moves), no atomics:
+//   bwd_dq_f32_mfma_kernel<D, KS>   4 waves, a wave owns 32 query rows (lane = row; Q, dO operands in registers) and one of
+//                        KS key shares: S^T = K Q^T and dP^T = V dO^T (accumulators start at -DELTA), dS^T = P (dP - DELTA)
+//                        in registers, dQ^T += K^T dS^T with the accumulator register as the step's operand; the KS partial
+//                        dQ of a row group are summed through LDS; dQ is added to the fp32 accumulator in whole rows.
+//   bwd_dkdv_f32_mfma_kernel<D>     4 waves, a wave owns 32 keys (lane = key; K, V operands and the dK^T, dV^T accumulators
+//                        in registers: one wave per SIMD), the block loops over the group's query heads and over 32-row
+//                        Q / dO tiles in double-buffered LDS: S = Q K^T, dP = dO V^T (accumulators start at -DELTA of
+//                        their rows), P and dS in registers, dV^T += dO^T P, dK^T += Q^T dS.
+template <int D, int KS>
+__global__ __launch_bounds__(256) void bwd_dq_f32_mfma_kernel(const BwdParams p) {
+    using L = F32Mfma<D, KS>;
+    constexpr int NW = L::NW, RG = L::RG, BM = L::BM, BN = L::BN, TILE = L::TILE;
+    constexpr int CPR = D / 4, RPI = 64 / CPR, NI = BN / (RPI * NW);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = w / KS, ks = w % KS;
+    const bool causal = p.flags & LTR_CAUSAL;
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    const int idx = blockIdx.x;
+    const int qt = n_qt - 1 - idx / (p.B * p.Hq);
+    const int bh = idx % (p.B * p.Hq);
+    const int b = bh / p.Hq, h = bh % p.Hq, hkv = h / p.n_rep;
+    const int row0 = qt * BM, my_row = row0 + rg * 32 + l32;
+    const bool row_ok = my_row < p.Sq;
+    const int my_pos = q_position(my_row, p.q_split, p.q_pos0[0], p.q_pos0[1]);
+    int blk_lo, blk_hi, w_lo, w_hi;
+    q_pos_range(row0, min(row0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], blk_lo, blk_hi);
+    {
+        const int wr0 = row0 + rg * 32, wr1 = min(wr0 + 32, p.Sq) - 1;
+        if (wr1 >= wr0) q_pos_range(wr0, wr1, p.q_split, p.q_pos0[0], p.q_pos0[1], w_lo, w_hi);
+        else { w_lo = 0x7fffffff; w_hi = -0x7fffffff; }
+    }
+    // operands of the lane's row: qreg[4g + j] = Q[row][8g + 4h + j], doreg likewise
+    float qreg[D / 2], doreg[D / 2];
+    float lse2 = INFINITY, dlt = 0.f;   // +inf: P = exp2(s - inf) = 0 for rows past the end and rows that saw no key
+    {
+        const int rs = min(my_row, p.Sq - 1);
+        const float *qp = (const float *)p.q + b * p.qs[0] + (long long)rs * p.qs[1] + h * p.qs[2];
+        const float *dop = (const float *)p.d_o + b * p.dos[0] + (long long)rs * p.dos[1] + h * p.dos[2];
+#pragma unroll
+        for (int g = 0; g < D / 8; g++) {
+            const f32x4 x = *(const f32x4 *)(qp + 8 * g + 4 * hh), y = *(const f32x4 *)(dop + 8 * g + 4 * hh);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                qreg[4 * g + j] = x[j];
+                doreg[4 * g + j] = y[j];
+            }
+        }
+        if (row_ok) {
+            const float lse_row = p.lse[((long long)b * p.Hq + h) * p.Sq + my_row];
+            lse2 = lse_row == -INFINITY ? INFINITY : lse_row * LTR_LOG2E;
+            dlt = p.delta[((long long)b * p.Hq + h) * p.Sq + my_row];
+        }
+    }
+    f32x16 dqacc[D / 32], ndlt;
+#pragma unroll
+    for (int r = 0; r < 16; r++) ndlt[r] = -dlt;
+#pragma unroll
+    for (int i = 0; i < D / 32; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dqacc[i][r] = 0.f;
+    const float c2 = p.scale * LTR_LOG2E;
+
+    int c = -1, t = 0, nt = 0;
+    int ld_sk = 0, ld_pos0 = 0;
+    const float *ld_kb = nullptr, *ld_vb = nullptr;
+    auto settle = [&]() {
+        while (c < p.n_chunks && t >= nt) {
+            c++;
+            t = 0;
+            if (c < p.n_chunks) {
+                ld_sk = p.chunk[c].sk;
+                ld_pos0 = p.chunk[c].pos0;
+                ld_kb = (const float *)p.chunk[c].k + b * p.ks[0] + hkv * p.ks[2];
+                ld_vb = (const float *)p.chunk[c].v + b * p.vs[0] + hkv * p.vs[2];
+                const int nvis = causal ? max(0, min(ld_sk, blk_hi - ld_pos0 + 1)) : ld_sk;
+                nt = (nvis + BN - 1) / BN;
+            }
+        }
+    };
+    settle();
+    const int st_row = lane / CPR, st_pc = lane % CPR;
+    int nx_sk = 0, nx_pos0 = 0, nx_key0 = 0;
+    auto gload = [&](int ti, int buf) {
+        nx_sk = ld_sk;
+        nx_pos0 = ld_pos0;
+        nx_key0 = ti * BN;
+        const unsigned Kd = lds_address(smem) + buf * L::BUF_BYTES, Vd = Kd + TILE * 4;
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const int row = RPI * (NI * w + i) + st_row;
+            const int key = min(ti * BN + row, ld_sk - 1);
+            const int chunk = st_pc ^ f32_swz(row);
+            global_to_lds_b128(ld_kb + ((long long)key * p.ks[1] + chunk * 4), Kd + RPI * (NI * w + i) * D * 4);
+            global_to_lds_b128(ld_vb + ((long long)key * p.vs[1] + chunk * 4), Vd + RPI * (NI * w + i) * D * 4);
+        }
+    };
+    bool have = c < p.n_chunks;
+    if (!have) return;              // no visible key: nothing to add to the accumulator (block-uniform)
+    gload(t, 0);
+    tile_barrier();
+    int par = 0;
+    while (have) {
+        const int sk = nx_sk, pos0 = nx_pos0, key0 = nx_key0 + 32 * ks;
+        const float *Ks = (const float *)(smem + par * L::BUF_BYTES) + 32 * ks * D, *Vs = Ks + TILE;
+        t++;
+        settle();
+        const bool have_next = c < p.n_chunks;
+        if (have_next) gload(t, par ^ 1);
+        if (key0 < sk && (!causal || pos0 + key0 <= w_hi)) {
+            f32x16 s, dp = ndlt;
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[r] = 0.f;
+            const float *krow = Ks + l32 * D, *vrow_ = Vs + l32 * D;
+            const int ksw = f32_swz(l32);
+#pragma unroll
+            for (int g = 0; g < D / 8; g++) {
+                const f32x4 kx = *(const f32x4 *)(krow + (((2 * g + hh) ^ ksw) << 2));
+                const f32x4 vx = *(const f32x4 *)(vrow_ + (((2 * g + hh) ^ ksw) << 2));
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[j], qreg[4 * g + j], s, 0, 0, 0);
+                    dp = __builtin_amdgcn_mfma_f32_32x32x2f32(vx[j], doreg[4 * g + j], dp, 0, 0, 0);
+                }
+            }
+            const bool need_mask = (key0 + 32 > sk) || (causal && (pos0 + key0 + 31 > w_lo));
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2);
+                if (need_mask) {
+                    const int key = key0 + 8 * (r / 4) + 4 * hh + (r % 4);
+                    const bool vis = key < sk && row_ok && (!causal || pos0 + key <= my_pos);
+                    pv = vis ? pv : 0.f;
+                }
+                s[r] = pv * dp[r];          // dS^T, key 8 (r / 4) + 4h + r % 4 of the sub-tile
+            }
+            // dQ^T += K^T dS^T: step r contracts the key of accumulator register r; lane (d = 32 db + l32, h) reads K[key][d]
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int krow_i = 8 * (r / 4) + 4 * hh + (r % 4);
+                const float *kr = Ks + krow_i * D + (l32 & 3);
+                const int sw = f32_swz(krow_i);
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    const float kx = kr[((8 * db + (l32 >> 2)) ^ sw) << 2];
+                    dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(kx, s[r], dqacc[db], 0, 0, 0);
+                }
+            }
+        }
+        tile_barrier();
+        par ^= 1;
+        have = have_next;
+    }
+    // sum of the KS partial dQ of a row group
+    if constexpr (KS > 1) {
+        float *part = (float *)(smem + L::PART_OFF);
+        if (ks > 0) {
+            float *mine = part + (size_t)(rg * (KS - 1) + ks - 1) * (L::PART_BYTES / 4);
+#pragma unroll
+            for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    f32x4 x;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] = dqacc[i][4 * r4 + e];
+                    *(f32x4 *)(mine + ((i * 4 + r4) * 64 + lane) * 4) = x;
+                }
+        }
+        __syncthreads();
+        if (ks > 0) return;
+        for (int k2 = 1; k2 < KS; k2++) {
+            const float *other = part + (size_t)(rg * (KS - 1) + k2 - 1) * (L::PART_BYTES / 4);
+#pragma unroll
+            for (int i = 0; i < D / 32; i++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    const f32x4 x = *(const f32x4 *)(other + ((i * 4 + r4) * 64 + lane) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) dqacc[i][4 * r4 + e] += x[e];
+                }
+        }
+    }
+    unsigned char *stage = smem + L::STAGE_OFF + rg * WaveStage<D>::BYTES;
+    constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;
+    const int wave_row0 = row0 + rg * 32, Sq = p.Sq;
+    const long long dqs1 = p.dqs[1];
+    float *dqp = (float *)p.dq + b * p.dqs[0] + h * p.dqs[2] + (long long)(wave_row0 + lane / LPR) * dqs1 + 4 * (lane % LPR);
+    wave_tile_rowmajor<D>(stage, lane, dqacc, p.scale, [&](int row, int, f32x4 val) {
+        if (wave_row0 + row < Sq) {
+            const f32x4 old = *(const f32x4 *)dqp;
+#pragma unroll
+            for (int e = 0; e < 4; e++) val[e] += old[e];
+            *(f32x4 *)dqp = val;
+        }
+        dqp += ROWS_PER_IT * dqs1;
+    });
+}
+
+template <int D>
+struct F32DkdvLds {
+    static constexpr int TILE = 32 * D;                          // floats per Q (or dO) tile of 32 rows
+    static constexpr int BUF_BYTES = 2 * TILE * 4 + 3 * 32 * 4;  // Q, dO, LSE * log2(e), -DELTA, row positions
+    static constexpr int STAGE_BYTES = 4 * WaveStage<D>::BYTES;
+    static constexpr int LDS = 2 * BUF_BYTES > STAGE_BYTES ? 2 * BUF_BYTES : STAGE_BYTES;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dkdv_f32_mfma_kernel(const BwdParams p) {
+    using L = F32DkdvLds<D>;
+    constexpr int BN = 128, BM = 32, TILE = L::TILE;
+    constexpr int CPR = D / 4, RPI = 64 / CPR, NI = BM / (RPI * 4);
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool causal = p.flags & LTR_CAUSAL;
+    // block -> (batch, kv head, chunk, 128-key tile)
+    const int P = p.B * p.Hkv;
+    const int pair = blockIdx.x % P;
+    int c = 0, kt = blockIdx.x / P;
+    for (; c < p.n_chunks; c++) {
+        const int n = (p.chunk[c].sk + BN - 1) / BN;
+        if (kt < n) break;
+        kt -= n;
+    }
+    if (c >= p.n_chunks) return;
+    const int b = pair / p.Hkv, hkv = pair % p.Hkv;
+    const int sk = p.chunk[c].sk, pos0 = p.chunk[c].pos0;
+    const int key0 = kt * BN, my_key = key0 + 32 * w + l32;
+    const bool key_ok = my_key < sk;
+    const int kpos = key_ok ? pos0 + my_key : BWD_KPOS_NONE;
+    const int blk_kpos_lo = pos0 + key0, w_kpos_lo = pos0 + key0 + 32 * w;
+    if (causal) {   // no query of this launch sees the block
+        int q_lo, q_hi;
+        q_pos_range(0, (int)p.Sq - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], q_lo, q_hi);
+        if (q_hi < blk_kpos_lo) return;
+    }
+    // operands of the lane's key: kreg[4g + j] = K[key][8g + 4h + j], vreg likewise
+    float kreg[D / 2], vreg[D / 2];
+    {
+        const int ksafe = min(my_key, sk - 1);
+        const float *kp = (const float *)p.chunk[c].k + b * p.ks[0] + (long long)ksafe * p.ks[1] + hkv * p.ks[2];
+        const float *vp = (const float *)p.chunk[c].v + b * p.vs[0] + (long long)ksafe * p.vs[1] + hkv * p.vs[2];
+#pragma unroll
+        for (int g = 0; g < D / 8; g++) {
+            f32x4 x = *(const f32x4 *)(kp + 8 * g + 4 * hh), y = *(const f32x4 *)(vp + 8 * g + 4 * hh);
+            if (!key_ok) x = y = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                kreg[4 * g + j] = x[j];
+                vreg[4 * g + j] = y[j];
+            }
+        }
+    }
+    f32x16 dkacc[D / 32], dvacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dkacc[i][r] = dvacc[i][r] = 0.f;
+    const float c2 = p.scale * LTR_LOG2E;
+
+    // walk over (query head of the group, 32-row q tile); tiles none of whose rows sees a key of the block are skipped
+    const int n_qt = (p.Sq + BM - 1) / BM, total = p.n_rep * n_qt;
+    auto visible = [&](int it) {
+        if (!causal) return true;
+        const int r0 = (it % n_qt) * BM;
+        int lo, hi;
+        q_pos_range(r0, min(r0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
+        return hi >= blk_kpos_lo;
+    };
+    auto next_visible = [&](int it) {
+        while (it < total && !visible(it)) it++;
+        return it;
+    };
+    const int st_row = lane / CPR, st_pc = lane % CPR;
+    auto gload = [&](int it, int buf) {
+        const int rep = it / n_qt, r0 = (it % n_qt) * BM, h = hkv * p.n_rep + rep;
+        const float *qp = (const float *)p.q + b * p.qs[0] + h * p.qs[2];
+        const float *dop = (const float *)p.d_o + b * p.dos[0] + h * p.dos[2];
+        const unsigned Qd = lds_address(smem) + buf * L::BUF_BYTES, dOd = Qd + TILE * 4;
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const int row = RPI * (NI * w + i) + st_row;
+            const int grow = min(r0 + row, p.Sq - 1);
+            const int chunk = st_pc ^ f32_swz(row);
+            global_to_lds_b128(qp + ((long long)grow * p.qs[1] + chunk * 4), Qd + RPI * (NI * w + i) * D * 4);
+            global_to_lds_b128(dop + ((long long)grow * p.dos[1] + chunk * 4), dOd + RPI * (NI * w + i) * D * 4);
+        }
+        // per-row scalars of the tile: LSE * log2(e) (+inf for rows past the end or without a visible key), -DELTA, position
+        float *st = (float *)(smem + buf * L::BUF_BYTES) + 2 * TILE;
+        if (tid < 96) {
+            const int r = tid & 31, row = r0 + r;
+            const bool ok = row < p.Sq;
+            const long long so = ((long long)b * p.Hq + h) * p.Sq + min(row, p.Sq - 1);
+            if (tid < 32) {
+                const float l = p.lse[so];
+                st[r] = (!ok || l == -INFINITY) ? INFINITY : l * LTR_LOG2E;
+            } else if (tid < 64) {
+                st[32 + r] = ok ? -p.delta[so] : 0.f;
+            } else {
+                ((int *)st)[64 + r] = !ok ? BWD_QPOS_NONE : causal ? q_position(row, p.q_split, p.q_pos0[0], p.q_pos0[1]) : BWD_QPOS_ALL;
+            }
+        }
+    };
+    int it = next_visible(0);
+    if (it < total) gload(it, 0);
+    tile_barrier();
+    int par = 0;
+    while (it < total) {
+        const int nxt = next_visible(it + 1);
+        if (nxt < total) gload(nxt, par ^ 1);
+        const float *Qs = (const float *)(smem + par * L::BUF_BYTES), *dOs = Qs + TILE;
+        const float *st = dOs + TILE;
+        // a wave whose 32 keys no row of the tile sees has nothing to add
+        int lo, hi;
+        {
+            const int r0 = (it % n_qt) * BM;
+            q_pos_range(r0, min(r0 + BM, p.Sq) - 1, p.q_split, p.q_pos0[0], p.q_pos0[1], lo, hi);
+        }
+        if (!causal || hi >= w_kpos_lo) {
+            f32x16 s, dp;
+            float lse2[16];
+            int qpos[16];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const f32x4 a = *(const f32x4 *)(st + 8 * g + 4 * hh), d4 = *(const f32x4 *)(st + 32 + 8 * g + 4 * hh);
+                const i32x4 q4 = *(const i32x4 *)((const int *)st + 64 + 8 * g + 4 * hh);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    lse2[4 * g + e] = a[e];
+                    dp[4 * g + e] = d4[e];      // the dP accumulator starts at -DELTA of its row
+                    qpos[4 * g + e] = q4[e];
+                    s[4 * g + e] = 0.f;
+                }
+            }
+            const float *qrow = Qs + l32 * D, *dorow = dOs + l32 * D;
+            const int rsw = f32_swz(l32);
+#pragma unroll
+            for (int g = 0; g < D / 8; g++) {
+                const f32x4 qx = *(const f32x4 *)(qrow + (((2 * g + hh) ^ rsw) << 2));
+                const f32x4 dx = *(const f32x4 *)(dorow + (((2 * g + hh) ^ rsw) << 2));
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    s = __builtin_amdgcn_mfma_f32_32x32x2f32(qx[j], kreg[4 * g + j], s, 0, 0, 0);
+                    dp = __builtin_amdgcn_mfma_f32_32x32x2f32(dx[j], vreg[4 * g + j], dp, 0, 0, 0);
+                }
+            }
+            // register r <-> tile row 8 (r / 4) + 4h + r % 4, lane <-> key: P and dS of the (row, key) pair
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float pv = __builtin_amdgcn_exp2f(s[r] * c2 - lse2[r]);
+                pv = kpos <= qpos[r] ? pv : 0.f;
+                s[r] = pv;
+                dp[r] = pv * dp[r];
+            }
+            // dV^T += dO^T P and dK^T += Q^T dS: step r contracts the row of accumulator register r; lane (d = 32 db + l32, h)
+            // reads dO[row][d] / Q[row][d]
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int trow = 8 * (r / 4) + 4 * hh + (r % 4);
+                const int sw = f32_swz(trow);
+                const float *dor = dOs + trow * D + (l32 & 3), *qr = Qs + trow * D + (l32 & 3);
+#pragma unroll
+                for (int db = 0; db < D / 32; db++) {
+                    const int off = ((8 * db + (l32 >> 2)) ^ sw) << 2;
+                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(dor[off], s[r], dvacc[db], 0, 0, 0);
+                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(qr[off], dp[r], dkacc[db], 0, 0, 0);
+                }
+            }
+        }
+        tile_barrier();
+        par ^= 1;
+        it = nxt;
+    }
+    // dK^T / dV^T of the wave's 32 keys: added to the fp32 accumulators in whole rows through the wave's staging area
+    unsigned char *stage = smem + w * WaveStage<D>::BYTES;
+    constexpr int LPR = D / 4, ROWS_PER_IT = 64 / LPR;
+    const int key_base = key0 + 32 * w;
+    auto add_rows = [&](const f32x16 (&acc)[D / 32], float mul, float *base, long long stride) {
+        float *gp = base + (long long)(key_base + lane / LPR) * stride + 4 * (lane % LPR);
+        wave_tile_rowmajor<D>(stage, lane, acc, mul, [&](int row, int, f32x4 val) {
+            if (key_base + row < sk) {
+                const f32x4 old = *(const f32x4 *)gp;
+#pragma unroll
+                for (int e = 0; e < 4; e++) val[e] += old[e];
+                *(f32x4 *)gp = val;
+            }
+            gp += ROWS_PER_IT * stride;
+        });
+    };
+    add_rows(dkacc, p.scale, p.chunk[c].dk + b * p.dks[0] + hkv * p.dks[2], p.dks[1]);
+    add_rows(dvacc, 1.f, p.chunk[c].dv + b * p.dvs[0] + hkv * p.dvs[2], p.dvs[1]);
+}
+
 // ------------------------------------------------------------------------------ host side
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -2478,7 +2878,21 @@ int enable_large_lds() {
               hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   F32Mfma<64, 2>::LDS) == hipSuccess &&
               hipFuncSetAttribute((const void *)fwd_f32_mfma_kernel<64, 4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  F32Mfma<64, 4>::LDS) == hipSuccess;
+                                  F32Mfma<64, 4>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_f32_mfma_kernel<128, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<128, 1>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_f32_mfma_kernel<128, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<128, 2>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_f32_mfma_kernel<64, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<64, 1>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_f32_mfma_kernel<64, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<64, 2>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dq_f32_mfma_kernel<64, 4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32Mfma<64, 4>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dkdv_f32_mfma_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32DkdvLds<128>::LDS) == hipSuccess &&
+              hipFuncSetAttribute((const void *)bwd_dkdv_f32_mfma_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  F32DkdvLds<64>::LDS) == hipSuccess;
     if (!ok) {
         (void)hipGetLastError();
         return LTR_ELAUNCH;
@@ -2614,6 +3028,7 @@ FwdPlan plan_fwd(int D, bool f32, unsigned flags, int B, int Hq, int Sq, int q_s
 
 // The same for the two backward kernels.
 struct BwdPlan {
+    int f32_ks;         // fp32: 0 = scalar kernels, else the key shares per row group of bwd_dq_f32_mfma_kernel
     bool wide_kv;       // dK/dV kernel: 256 keys per block (two 32-key halves per wave, head dim 64)
     int keys_per_block;
     long long kv_tiles; // key blocks over all chunks of one (batch, kv head)
@@ -2625,14 +3040,26 @@ struct BwdPlan {
 BwdPlan plan_bwd(int D, bool f32, unsigned flags, int B, int Hq, int Hkv, int Sq, int q_split, const int *q_pos0, const ChunkDev *chunk,
                  int n_chunks) {
     BwdPlan pl;
+    pl.f32_ks = 0;
     if (f32) {
         pl.wide_kv = pl.wide_q = false;
-        pl.keys_per_block = 64;
+        if (flags & LTR_BWD_F32_SCALAR) {
+            pl.keys_per_block = 64;
+            pl.dq_rows = 64;
+        } else {
+            // matrix-pipe kernels: 128 keys per dK/dV block; the dQ kernel sized like the fp32 forward (see plan_fwd)
+            const int cus = device_cus();
+            const int max_ks = D == 64 ? 4 : 2;
+            int ks = 1;
+            while (ks < max_ks && (long long)((Sq + 128 / ks - 1) / (128 / ks)) * B * Hq < cus) ks *= 2;
+            pl.f32_ks = ks;
+            pl.keys_per_block = 128;
+            pl.dq_rows = 128 / ks;
+        }
         pl.kv_tiles = 0;
-        for (int c = 0; c < n_chunks; c++) pl.kv_tiles += (chunk[c].sk + 63) / 64;
+        for (int c = 0; c < n_chunks; c++) pl.kv_tiles += (chunk[c].sk + pl.keys_per_block - 1) / pl.keys_per_block;
         pl.kv_blocks = pl.kv_tiles * B * Hkv;
-        pl.dq_rows = 64;
-        pl.dq_qtiles = pl.dq_slots = (Sq + 63) / 64;
+        pl.dq_qtiles = pl.dq_slots = (Sq + pl.dq_rows - 1) / pl.dq_rows;
         pl.dq_blocks = (long long)pl.dq_qtiles * B * Hq;
         return pl;
     }
@@ -2872,8 +3299,9 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     if (a->B <= 0 || a->Hq <= 0 || a->Hkv <= 0 || a->Sq <= 0 || a->Hq % a->Hkv) return LTR_EINVAL;
     if (a->n_chunks < 1 || a->n_chunks > LTR_MAX_CHUNKS) return LTR_EINVAL;
     if (flags & ~(LTR_CAUSAL | LTR_NO_DQ | LTR_NO_DKDV | LTR_DQ_BF16 | LTR_DELTA_FROM_O | LTR_DKDV_BF16 | LTR_ROPE_DQ | LTR_DKDV_KEYS_128 |
-                  LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_256 | LTR_DQ_ROWS_512))
+                  LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_256 | LTR_DQ_ROWS_512 | LTR_BWD_F32_SCALAR))
         return LTR_EINVAL;
+    if ((flags & LTR_BWD_F32_SCALAR) && a->io_dtype != LTR_F32) return LTR_EUNSUP;
     if ((flags & LTR_DKDV_KEYS_128) && (flags & LTR_DKDV_KEYS_256)) return LTR_EINVAL;
     if ((flags & LTR_DQ_ROWS_256) && (flags & LTR_DQ_ROWS_512)) return LTR_EINVAL;
     const bool fused_delta = flags & LTR_DELTA_FROM_O;
@@ -2963,6 +3391,24 @@ int bwd_launch(const ltr_attn_bwd_args *a, unsigned flags, bool use_scratch, voi
     p.tiles_total = (int)pl.kv_tiles;
     p.n_slots = pl.dq_slots;
     hipStream_t st = (hipStream_t)stream;
+    if (f32 && pl.f32_ks) {   // fp32 on the matrix pipe
+        rc = enable_large_lds();
+        if (rc) return rc;
+        if (do_dq) {
+            if (a->D == 128)
+                rc = pl.f32_ks == 1 ? launch((const void *)bwd_dq_f32_mfma_kernel<128, 1>, pl.dq_blocks, 256, F32Mfma<128, 1>::LDS, st, p)
+                                    : launch((const void *)bwd_dq_f32_mfma_kernel<128, 2>, pl.dq_blocks, 256, F32Mfma<128, 2>::LDS, st, p);
+            else
+                rc = pl.f32_ks == 1   ? launch((const void *)bwd_dq_f32_mfma_kernel<64, 1>, pl.dq_blocks, 256, F32Mfma<64, 1>::LDS, st, p)
+                     : pl.f32_ks == 2 ? launch((const void *)bwd_dq_f32_mfma_kernel<64, 2>, pl.dq_blocks, 256, F32Mfma<64, 2>::LDS, st, p)
+                                      : launch((const void *)bwd_dq_f32_mfma_kernel<64, 4>, pl.dq_blocks, 256, F32Mfma<64, 4>::LDS, st, p);
+            if (rc) return rc;
+        }
+        if (do_dkdv)
+            rc = a->D == 128 ? launch((const void *)bwd_dkdv_f32_mfma_kernel<128>, pl.kv_blocks, 256, F32DkdvLds<128>::LDS, st, p)
+                             : launch((const void *)bwd_dkdv_f32_mfma_kernel<64>, pl.kv_blocks, 256, F32DkdvLds<64>::LDS, st, p);
+        return rc;
+    }
     if (f32) {
         if (do_dq) {
             rc = a->D == 128 ? launch((const void *)bwd_dq_f32_kernel<128>, pl.dq_blocks, 64, 0, st, p)
@@ -3046,8 +3492,13 @@ extern "C" int ltr_attn_plan(const ltr_attn_bwd_args *a, ltr_attn_plan_t *out) {
     if (f32) {
         if (f.f32_ks) snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_f32_mfma_kernel<%d, %d>", a->D, f.f32_ks);
         else snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_f32_kernel<%d>", a->D);
-        snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_f32_kernel<%d>", a->D);
-        snprintf(out->dkdv_kernel, sizeof(out->dkdv_kernel), "bwd_dkdv_f32_kernel<%d, *>", a->D);
+        if (b.f32_ks) {
+            snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_f32_mfma_kernel<%d, %d>", a->D, b.f32_ks);
+            snprintf(out->dkdv_kernel, sizeof(out->dkdv_kernel), "bwd_dkdv_f32_mfma_kernel<%d>", a->D);
+        } else {
+            snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_f32_kernel<%d>", a->D);
+            snprintf(out->dkdv_kernel, sizeof(out->dkdv_kernel), "bwd_dkdv_f32_kernel<%d, *>", a->D);
+        }
     } else {
         snprintf(out->fwd_kernel, sizeof(out->fwd_kernel), "fwd_bf16_kernel<%d, %d>", a->D, f.wide ? 2 : 1);
         snprintf(out->dq_kernel, sizeof(out->dq_kernel), "bwd_dq_kernel<%d, %d>", a->D, b.wide_q ? 2 : 1);

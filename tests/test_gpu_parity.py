@@ -219,6 +219,48 @@ def test_config1_fp32_ring_fwd_bwd(ltr):
     _grads_case(ltr, 2, 8, 8, 64, 1024, 4, "contiguous", True, 0, dtype=torch.float32)
 
 
+@pytest.mark.parametrize("D,B,Hq,Hkv,Sq,q_pos,split,chunks,causal", [
+    (64, 2, 8, 8, 256, (768, 768), None, [(768, 256), (512, 256), (256, 256), (0, 256)], True),     # config 1, rank 3: 4 key shares
+    (64, 4, 16, 4, 300, (100, 900), 130, [(0, 200), (200, 333), (533, 700)], True),                 # ragged, GQA, two-segment rows
+    (64, 2, 16, 16, 1024, (0, 0), None, [(0, 1024)], True),                                          # one key share
+    (128, 1, 4, 2, 200, (56, 56), None, [(0, 100), (100, 156)], True),
+    (128, 4, 16, 4, 520, (0, 0), None, [(0, 260), (260, 300)], False),
+])
+def test_fp32_backward_on_the_matrix_pipe(ltr, D, B, Hq, Hkv, Sq, q_pos, split, chunks, causal):
+    """The fp32 backward on v_mfma_f32_32x32x2_f32 (bwd_dq_f32_mfma_kernel in its key-share instantiations,
+    bwd_dkdv_f32_mfma_kernel) against dense fp64 autograd to 1e-4 relative per tensor, and against the scalar fp32 kernels
+    (LTR_BWD_F32_SCALAR); accumulation over two calls (the accumulators are added to, not overwritten)."""
+    lens, pos0 = [n for _, n in chunks], [p0 for p0, _ in chunks]
+    plan = ltr.attn_plan(B, Hq, Hkv, D, Sq, lens, pos0, q_pos, split, causal, dtype=torch.float32)
+    assert plan["dq"]["kernel"].startswith("bwd_dq_f32_mfma_kernel") and plan["dkdv"]["kernel"] == "bwd_dkdv_f32_mfma_kernel<%d>" % D
+    g = torch.Generator().manual_seed(4100 + Sq + D)
+    sp = Sq if split is None else split
+    qpos = torch.cat([torch.arange(sp) + q_pos[0], torch.arange(Sq - sp) + q_pos[1]])
+    q, do = _randn((B, Sq, Hq, D), g, torch.float32), _randn((B, Sq, Hq, D), g, torch.float32)
+    kbuf, vbuf = _randn((B, sum(lens), Hkv, D), g, torch.float32), _randn((B, sum(lens), Hkv, D), g, torch.float32)
+    kpos = torch.cat([torch.arange(n) + p0 for p0, n in chunks])
+    ro, rlse, rdq, rdk, rdv = orc.dense_attention_grads(q, kbuf, vbuf, do, qpos, kpos, causal)
+    qd, dod, kd, vd = q.cuda(), do.cuda(), kbuf.cuda(), vbuf.cuda()
+    offs = [sum(lens[:i]) for i in range(len(lens))]
+    ks = [kd[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+    vs = [vd[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+    o, lse = ltr.attn_fwd(qd, ks, vs, pos0, q_pos, split, causal)
+    delta = ltr.attn_delta(o, dod)
+    res = {}
+    for scalar in (False, True):
+        dq = torch.zeros_like(qd)
+        dk, dv = torch.zeros_like(kd), torch.zeros_like(vd)
+        dks = [dk[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+        dvs = [dv[:, o_:o_ + n_] for o_, n_ in zip(offs, lens)]
+        for _ in range(2):      # two calls: every gradient must come out doubled
+            ltr.attn_bwd_accumulate(qd, dod, lse, delta, ks, vs, pos0, dq, dks, dvs, q_pos, split, causal, f32_scalar=scalar)
+        res[scalar] = (dq.cpu() / 2, dk.cpu() / 2, dv.cpu() / 2)
+    for got, ref in zip(res[False], (rdq, rdk, rdv)):
+        assert _rel(got, ref) < 1e-4
+    for a, b in zip(res[False], res[True]):
+        assert _rel(a, b) < 2e-5
+
+
 def test_fp32_gqa_zigzag_d128_fwd_bwd(ltr):
     _grads_case(ltr, 1, 4, 2, 128, 512, 4, "zigzag", True, 5, dtype=torch.float32)
 

@@ -110,10 +110,13 @@ def test_plan_names_the_kernels_and_follows_the_hints():
     assert _plan(L, lib, 64, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_DQ_ROWS_512 | L.LTR_DQ_ROWS_256)[0] == -1
     assert _plan(L, lib, 96, 1, 4, 4, 512, [(512, 0)])[0] == -2
     rc, pl = _plan(L, lib, 64, 2, 8, 8, 1024, [(256, 0)] * 4, dtype=L.LTR_F32)    # config 1's shape, scalar fp32 kernels
-    assert rc == 0 and pl.fwd_kernel == b"fwd_f32_mfma_kernel<64, 2>" and pl.fwd_rows == 64 and pl.dkdv_blocks == 4 * 4 * 16
-    assert pl.dq_kernel == b"bwd_dq_f32_kernel<64>"
-    rc, pl = _plan(L, lib, 64, 2, 8, 8, 1024, [(256, 0)] * 4, dtype=L.LTR_F32, flags=L.LTR_FWD_F32_SCALAR)
+    assert rc == 0 and pl.fwd_kernel == b"fwd_f32_mfma_kernel<64, 2>" and pl.fwd_rows == 64
+    assert pl.dq_kernel == b"bwd_dq_f32_mfma_kernel<64, 2>" and pl.dq_rows == 64
+    assert pl.dkdv_kernel == b"bwd_dkdv_f32_mfma_kernel<64>" and pl.dkdv_keys == 128 and pl.dkdv_blocks == 4 * 2 * 16
+    rc, pl = _plan(L, lib, 64, 2, 8, 8, 1024, [(256, 0)] * 4, dtype=L.LTR_F32, flags=L.LTR_FWD_F32_SCALAR | L.LTR_BWD_F32_SCALAR)
     assert rc == 0 and pl.fwd_kernel == b"fwd_f32_kernel<64>" and pl.fwd_rows == 64
+    assert pl.dq_kernel == b"bwd_dq_f32_kernel<64>" and pl.dkdv_keys == 64 and pl.dkdv_blocks == 4 * 4 * 16
+    assert _plan(L, lib, 64, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_BWD_F32_SCALAR)[0] == 0       # the plan ignores it for bf16
 
 
 def test_validation_without_gpu():
