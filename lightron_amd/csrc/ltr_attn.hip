@@ -3468,6 +3468,7 @@ extern "C" int ltr_attn_plan(const ltr_attn_bwd_args *a, ltr_attn_plan_t *out) {
     if ((flags & LTR_FWD_ROWS_256) && (flags & LTR_FWD_ROWS_512)) return LTR_EINVAL;
     const bool f32 = a->io_dtype == LTR_F32;
     if ((flags & (LTR_DKDV_KEYS_256 | LTR_DQ_ROWS_512 | LTR_FWD_ROWS_512)) && (a->D != 64 || f32)) return LTR_EUNSUP;
+    if ((flags & (LTR_FWD_F32_SCALAR | LTR_BWD_F32_SCALAR)) && !f32) return LTR_EUNSUP;
     ChunkDev chunk[LTR_MAX_CHUNKS];
     for (int c = 0; c < a->n_chunks; c++) {
         const ltr_kv_chunk &ch = a->chunk[c];

@@ -116,7 +116,7 @@ def test_plan_names_the_kernels_and_follows_the_hints():
     rc, pl = _plan(L, lib, 64, 2, 8, 8, 1024, [(256, 0)] * 4, dtype=L.LTR_F32, flags=L.LTR_FWD_F32_SCALAR | L.LTR_BWD_F32_SCALAR)
     assert rc == 0 and pl.fwd_kernel == b"fwd_f32_kernel<64>" and pl.fwd_rows == 64
     assert pl.dq_kernel == b"bwd_dq_f32_kernel<64>" and pl.dkdv_keys == 64 and pl.dkdv_blocks == 4 * 4 * 16
-    assert _plan(L, lib, 64, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_BWD_F32_SCALAR)[0] == 0       # the plan ignores it for bf16
+    assert _plan(L, lib, 64, 1, 4, 4, 512, [(512, 0)], flags=L.LTR_BWD_F32_SCALAR)[0] == -2      # fp32 only, as in the launches
 
 
 def test_validation_without_gpu():
