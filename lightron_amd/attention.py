@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 import threading
 from typing import List, Optional, Sequence, Tuple
 
@@ -543,6 +544,27 @@ class SingleChunkAttentionFunction(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+# The single-chunk bf16 call has two host sides over the same two C-ABI calls: a C++ autograd node (_ltr_node.so, built by
+# lightron_amd.build: the backward then runs on the autograd thread without the interpreter) and SingleChunkAttentionFunction
+# (Python).  The C++ node is used when it has been built for this ABI version and the library is the in-tree one.
+USE_CPP_NODE = True
+_node = None
+
+
+def _cpp_node():
+    global _node
+    if _node is None:
+        _node = False
+        if not os.environ.get("LTR_ATTN_LIB"):        # the node is linked against the in-tree library
+            try:
+                from . import _ltr_node
+                if _ltr_node.abi_version() == _lib.LTR_ABI_VERSION:
+                    _node = _ltr_node
+            except (ImportError, OSError):       # not built, or built against another torch: the Python node serves
+                pass
+    return _node
+
+
 _warned_pad = False
 
 
@@ -597,6 +619,12 @@ def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, sca
             and q.is_cuda and ks[0].is_cuda and vs[0].is_cuda):
         if isinstance(q_pos0, (tuple, list)):
             q_pos0 = (int(q_pos0[0]), int(q_pos0[1]))
+        node = _cpp_node() if USE_CPP_NODE else None
+        if node:
+            qa, qb = q_pos0 if isinstance(q_pos0, tuple) else (q_pos0, q_pos0)
+            o, lse = node.single_chunk(q, ks[0], vs[0], int(k_pos0[0]), qa, qb, q.shape[1] if q_split is None else q_split, bool(causal),
+                                       scale if scale is not None else 1.0 / math.sqrt(q.shape[3]), _stream_ptr(q.device), q_rope)
+            return o, lse
         return SingleChunkAttentionFunction.apply(q, ks[0], vs[0], (int(k_pos0[0]), q_pos0, q_split, bool(causal), scale, q_rope))
     if kv_grad_acc is not None:
         dk_accs, dv_accs = kv_grad_acc

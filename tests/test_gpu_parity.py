@@ -136,6 +136,42 @@ def test_fp32_forward_on_the_matrix_pipe(ltr, D, B, Hq, Hkv, Sq, q_pos, split, c
     assert (o - o_sc).abs().max() < 2e-5
 
 
+@pytest.mark.parametrize("with_rope", [False, True])
+def test_single_chunk_host_sides_agree(ltr, with_rope):
+    """The single-chunk bf16 call through the C++ autograd node (_ltr_node.so) and through the Python autograd Function:
+    same two C-ABI calls, so O, LSE and all three gradients must be bit-identical; GQA, strided [B,H,S,D] views, a
+    non-contiguous dO, with and without the fused RoPE prologue; and the result against the dense oracle."""
+    from lightron_amd import attention as A
+    assert A._cpp_node(), "the C++ autograd node has not been built (python -m lightron_amd.build)"
+    g = torch.Generator().manual_seed(91)
+    B, S, Hq, Hkv, D = 2, 200, 8, 2, 64
+    q = _randn((B, Hq, S, D), g, torch.bfloat16).transpose(1, 2)
+    k = _randn((B, Hkv, S, D), g, torch.bfloat16).transpose(1, 2)
+    v = _randn((B, S, Hkv, D), g, torch.bfloat16)
+    do = _randn((B, Hq, S, D), g, torch.bfloat16).transpose(1, 2)
+    table = ltr.rope_table(ltr.precompute_freqs_cis(D, S, device="cuda")) if with_rope else None
+    res = []
+    for use_cpp in (True, False):
+        A.USE_CPP_NODE = use_cpp
+        try:
+            qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+            o, lse = ltr.block_attention(qd, [kd], [vd], [0], 0, None, causal=True, q_rope=table)
+            assert type(o.grad_fn).__name__ == ("CppFunction" if use_cpp else "SingleChunkAttentionFunctionBackward")
+            assert ("SingleChunkNode" in o.grad_fn.name()) == use_cpp
+            o.backward(do.cuda())
+            res.append((o.detach(), lse, qd.grad, kd.grad, vd.grad))
+        finally:
+            A.USE_CPP_NODE = True
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    if not with_rope:
+        pos = torch.arange(S)
+        ro, rlse, rdq, rdk, rdv = orc.dense_attention_grads(q.float(), k.float(), v.float(), do.float(), pos, pos, True, dtype=torch.float32)
+        o, lse, dq, dk, dv = (x.cpu() for x in res[0])
+        assert (o.float() - ro).abs().max() < O_TOL_BF16 and (lse - rlse).abs().max() < LSE_TOL_BF16
+        assert _rel(dq, rdq) < GRAD_RTOL_BF16 and _rel(dk, rdk) < GRAD_RTOL_BF16 and _rel(dv, rdv) < GRAD_RTOL_BF16
+
+
 def test_config2_shape_scaled_multi_chunk_bf16(ltr):
     """Config 2 at reduced B/H: last rank's Q chunk of 1024 against 8 KV chunks of 1024, bf16, causal,
     inputs N(0,1)*0.5, fused and step-wise (merge epilogue) paths."""
