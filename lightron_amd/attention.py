@@ -354,11 +354,13 @@ class BlockAttentionFunction(torch.autograd.Function):
         # fused RoPE prologue: the kernel rotates q on load and hands the rotated q back for the backward
         q_rot = torch.empty(q.shape, dtype=q.dtype, device=q.device) if q_rope is not None else None
         if stepwise:
-            # one launch per KV chunk, merged in the epilogue into an fp32 running (O, LSE)
-            o, lse = attn_fwd(q, ks[:1], vs[:1], k_pos0[:1], q_pos0, q_split, causal, scale, out_dtype=torch.float32,
+            # one launch per ring step, merged in the epilogue into an fp32 running (O, LSE); a step brings `g` chunks of the
+            # table (1, or the two half-chunks of a zig-zag rank chunk: stepwise = 2)
+            g = 1 if stepwise is True else int(stepwise)
+            o, lse = attn_fwd(q, ks[:g], vs[:g], k_pos0[:g], q_pos0, q_split, causal, scale, out_dtype=torch.float32,
                               q_rope=q_rope, q_rot_out=q_rot)
-            for i in range(1, n_chunks):
-                attn_fwd(q, ks[i:i + 1], vs[i:i + 1], k_pos0[i:i + 1], q_pos0, q_split, causal, scale,
+            for i in range(g, n_chunks, g):
+                attn_fwd(q, ks[i:i + g], vs[i:i + g], k_pos0[i:i + g], q_pos0, q_split, causal, scale,
                          out=o, lse=lse, merge=True, q_rope=q_rope)
             if (out_dtype or q.dtype) != torch.float32:
                 o = o.to(out_dtype or q.dtype)
@@ -605,7 +607,8 @@ def _padded_head_dim(q, ks, vs, k_pos0, q_pos0, q_split, causal, scale, stepwise
 
 def block_attention(q, ks, vs, k_pos0, q_pos0=0, q_split=None, causal=False, scale=None, stepwise=False,
                     out_dtype=None, kv_grad_acc=None, q_rope=None):
-    """Differentiable entry: returns (O, LSE).  q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table indexed by global
+    """Differentiable entry: returns (O, LSE).  stepwise: False = one launch over the whole chunk table; True or an int g = one
+    launch per g chunks, the partial (O, LSE) merged in the kernel's epilogue (the call pattern of a ring).  q_rope: fp32 [n_pos, D/2, 2] (cos, sin) table indexed by global
     position (layers.rope_table of precompute_freqs_cis): q is un-rotated, the forward kernel's prologue applies RoPE
     to it and the dQ kernel's epilogue the conjugate rotation, so no separate pass touches q or dQ (bf16 only).  ks are
     taken as given: rotate K once beforehand (apply_rotary_emb), it is read by every q block.  kv_grad_acc = (dk_accs, dv_accs), fp32 tensors shaped like ks / vs:

@@ -144,7 +144,10 @@ def ring_attention_with_lse(local_q, local_k, local_v, cp_group) -> Tuple[torch.
     ks, vs, pos, grad_acc = _chunk_table(ring, local_k, local_v, S_local)
     if grad_acc is not None and ring.kv[ring.rank] is None:
         raise RuntimeError("kv_grads needs the ring's own chunk in LocalRing.kv (entry %d is None)" % ring.rank)
-    o, lse = block_attention(local_q, ks, vs, pos, q_pos0, q_split, ring.causal, None, ring.stepwise,
+    # a ring step delivers one rank's chunk: one table entry, or the two half-chunks of a zig-zag chunk in ONE launch (the
+    # dK/dV and forward kernels then see twice the keys per launch: a block for every CU where a half-chunk leaves half idle)
+    step = (2 if ring.layout == "zigzag" else 1) if ring.stepwise else False
+    o, lse = block_attention(local_q, ks, vs, pos, q_pos0, q_split, ring.causal, None, step,
                              ring.out_dtype, grad_acc)
     return o, lse
 
