@@ -1521,6 +1521,26 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
     __syncthreads();
 
     const int st_row = lane / CPR, st_pc = lane % CPR;   // this lane's place inside a 1 KB LDS-direct load
+    // Per-lane element offsets of this lane's pieces of a Q / dO tile (unmasked tiles: row and chunk do not depend on the
+    // tile) and the bases of the current q head: a step then adds one scalar product per tensor instead of redoing the
+    // 64-bit address arithmetic of (batch, head, row).
+    unsigned offq[NI], offdo[NI];
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        const int row = RPI * (NI * w + i) + st_row;
+        const int chunk = st_pc ^ lds_swz<D>(row);
+        offq[i] = (unsigned)(row * (int)p.qs[1] + chunk * 8);
+        offdo[i] = (unsigned)(row * (int)p.dos[1] + chunk * 8);
+    }
+    const __bf16 *qp_head = nullptr, *dop_head = nullptr;
+    const float *sp_head = nullptr;   // LSE (wave 0) or DELTA - BM (wave 1) of the head's rows, indexed by row0 + tid
+    auto set_head = [&](int rep) __attribute__((always_inline)) {
+        const int h = hkv * p.n_rep + rep;
+        qp_head = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
+        dop_head = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
+        const long long so = ((long long)b * p.Hq + h) * p.Sq;
+        sp_head = w == 0 ? p.lse + so : p.delta + so - BM;
+    };
     const float st_mul = tid < BM ? -1.f / p.scale : -1.f;  // threads 0..63 stage -LSE/scale, 64..127 stage -DELTA
     float sld = 0.f;      // raw LSE / DELTA value in flight; scaled when it is written to LDS
     bool sld_ok = true;
@@ -1541,6 +1561,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
             if (++li_ >= cnt) {
                 li_ = 0;
                 if (++rep >= p.n_rep) return false;
+                set_head(rep);
             }
             qt = __builtin_amdgcn_readfirstlane((int)pre);
             pre = list[li_ + 1 < cnt ? li_ + 1 : 0];
@@ -1551,23 +1572,28 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         // l % CPR of row l / CPR, fetching the logical chunk the swizzle places there.  Rows past the end of Q
         // repeat its last row (they are masked).  LSE and DELTA go through a register of threads 0..127.
         auto gload = [&](int rep, int qt, int buf) {
-            const int h = hkv * p.n_rep + rep;
             const int row0 = qt * BM;
             sld_row0 = row0;
-            const __bf16 *qp = (const __bf16 *)p.q + b * p.qs[0] + h * p.qs[2];
-            const __bf16 *dop = (const __bf16 *)p.d_o + b * p.dos[0] + h * p.dos[2];
-            const long long so = ((long long)b * p.Hq + h) * p.Sq + row0;
-            const float *sp = tid < BM ? p.lse + so : p.delta + so - BM;   // indexed by tid below
             const unsigned Qd = lds_address(smem) + buf * L::BUF_BYTES, dOd = Qd + L::TILE * 2;   // LDS byte addresses
+            if (!MASK) {
+                const unsigned tq = (unsigned)(row0 * (int)p.qs[1]), tdo = (unsigned)(row0 * (int)p.dos[1]);
 #pragma unroll
-            for (int i = 0; i < NI; i++) {
-                const int row = RPI * (NI * w + i) + st_row;
-                const int grow = MASK ? min(row0 + row, p.Sq - 1) : row0 + row;
-                const int chunk = st_pc ^ lds_swz<D>(row);
-                global_to_lds_b128(qp + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D * 2);
-                global_to_lds_b128(dop + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D * 2);
+                for (int i = 0; i < NI; i++) {
+                    global_to_lds_b128(qp_head + (unsigned long long)(tq + offq[i]), Qd + RPI * (NI * w + i) * D * 2);
+                    global_to_lds_b128(dop_head + (unsigned long long)(tdo + offdo[i]), dOd + RPI * (NI * w + i) * D * 2);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NI; i++) {
+                    const int row = RPI * (NI * w + i) + st_row;
+                    const int grow = min(row0 + row, p.Sq - 1);
+                    const int chunk = st_pc ^ lds_swz<D>(row);
+                    global_to_lds_b128(qp_head + (long long)(grow * (int)p.qs[1] + chunk * 8), Qd + RPI * (NI * w + i) * D * 2);
+                    global_to_lds_b128(dop_head + (long long)(grow * (int)p.dos[1] + chunk * 8), dOd + RPI * (NI * w + i) * D * 2);
+                }
             }
             if (tid < 2 * BM) {
+                const float *sp = sp_head + row0;
                 if (!MASK) {
                     sld = sp[tid];
                 } else {
@@ -1596,6 +1622,7 @@ __global__ __launch_bounds__(512) void bwd_dkdv_kernel(const BwdParams p) {
         for (int k = 0; k < KW; k++) kpos[k] = key_ok[k] ? pos0 + my_key[k] : BWD_KPOS_NONE;
         if (cnt == 0) return;
         int rep = 0, qt = 0;
+        set_head(0);
         advance(rep, qt);
         __syncthreads();   // the previous pass has finished reading LDS
         gload(rep, qt, 0);
