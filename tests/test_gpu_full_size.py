@@ -1,4 +1,4 @@
-"""Full-size GPU tests of BASELINE configs 2-5.  The dense oracle does not finish in seconds at
+"""Full-size GPU tests of the benchmark configs 2-5.  The dense oracle does not finish in seconds at
 these sizes, so each test checks sampled query rows (O, LSE, dQ) and sampled keys (dK, dV)
 against the oracle's closed form restricted to those rows / keys (fp64, CPU, same seeded bf16
 inputs), plus size-independent identities: sum_j dV_j = sum_i dO_i per kv group (softmax rows

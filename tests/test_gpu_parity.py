@@ -51,7 +51,7 @@ def test_fwd_single_chunk_bf16(ltr, D, Hq, Hkv, Sq, Sk, causal):
 
 
 def test_config1_fp32_ring_four_ranks(ltr):
-    """BASELINE config 1: B=2 H=8 S=1024 as 4 x 256, D=64, fp32, causal, seed 0, forward."""
+    """benchmark config 1: B=2 H=8 S=1024 as 4 x 256, D=64, fp32, causal, seed 0, forward."""
     g = torch.Generator().manual_seed(0)
     q, k, v = (torch.randn((2, 8, 1024, 64), generator=g) for _ in range(3))   # [B,H,S,D] as stated
     qs, ks, vs = (x.transpose(1, 2) for x in (q, k, v))                        # views [B,S,H,D]

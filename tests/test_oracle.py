@@ -41,7 +41,7 @@ def test_reference_acceptance_noncausal_vs_sdpa():
 
 
 def test_config1_causal_vs_sdpa_fp64():
-    # BASELINE config 1: B=2 H=8 S=1024 (4x256) D=64 fp32 causal, seed 0
+    # benchmark config 1: B=2 H=8 S=1024 (4x256) D=64 fp32 causal, seed 0
     g = torch.Generator().manual_seed(0)
     q, k, v = (torch.randn((2, 1024, 8, 64), generator=g) for _ in range(3))
     o, lse = _ring_all_ranks(q, k, v, 4, causal=True)
